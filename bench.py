@@ -1,0 +1,203 @@
+#!/usr/bin/env python3
+"""Benchmark of the packed-int4 linear-layer GEMM on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-decode]
+
+A step is one GEMM launch C[MxN] = A[MxK] * B[NxK]^T through the library's C ABI
+(int4linear_gemm_s4s4s32, asynchronous, on torch's current stream).  The workload is
+the square M = N = K = 8192 case the headline metric is quoted on; inputs are synthetic
+seeded s4 values already resident in HBM when the clock starts.  Operand sets rotate
+through more memory than L2 plus the 256 MB Infinity Cache, so no launch finds its
+operands cached by the previous one (the reference flushes L2 before every timed launch,
+test/benchmark.cu:77-96).  Throughput = 2*M*N*K / time (test/benchmark.cu:112-115).
+
+One JSON line is printed.  Besides the whole-run figure it carries
+  roofline      the GEMM kernel's own rate (HIP events around the timed launches on the
+                launch stream) against the int8 MFMA dense peak,
+  decode        the skinny-M weight-streaming kernel at M = 16 against HBM bandwidth,
+  cpu_baseline  the CPU oracle's loop nest timed on this host's cores on a row sample.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+INT8_MFMA_PEAK_TOPS = 5000.0   # MI355X dense int8, published
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+
+M = N = K = 8192
+DECODE_SHAPES = [(16, 4096, 4096), (16, 14336, 4096), (16, 4096, 14336)]
+
+
+def packed_random(torch, rows: int, k: int, seed: int):
+    """rows x k/2 bytes of uniform s4 pairs: every byte value 0..255 equally likely is
+    exactly two independent uniform nibbles in [-8, 7]."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    return torch.randint(0, 256, (rows, k // 2), dtype=torch.uint8, device="cuda", generator=g)
+
+
+def time_launches(torch, launch, sets, steps: int, warmup: int):
+    """Average milliseconds per launch: `warmup` untimed, then exactly `steps` timed
+    launches bracketed by a device synchronisation and a HIP event pair on the stream."""
+    for i in range(warmup):
+        launch(sets[i % len(sets)])
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for i in range(steps):
+        launch(sets[i % len(sets)])
+    stop.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    return start.elapsed_time(stop) / steps, wall_ms / steps
+
+
+def bench_gemm(torch, lib, steps: int, warmup: int):
+    # 3 operand sets x (32 + 32 + 256 MiB) = 960 MiB > L2 + Infinity Cache.
+    sets = []
+    for s in range(3):
+        a = packed_random(torch, M, K, 1000 + s)
+        b = packed_random(torch, N, K, 2000 + s)
+        c = torch.empty((M, N), dtype=torch.int32, device="cuda")
+        sets.append((a, b, c))
+
+    def launch(t):
+        lib.gemm_s4s4s32(t[0], t[1], t[2], M, N, K)
+
+    ev_ms, wall_ms = time_launches(torch, launch, sets, steps, warmup)
+    return ev_ms, wall_ms
+
+
+def bench_decode(torch, lib, steps: int, warmup: int):
+    out = []
+    for (m, n, k) in DECODE_SHAPES:
+        wbytes = n * k // 2
+        nsets = max(4, (768 << 20) // wbytes + 1)   # rotate through > 768 MiB of weights
+        x = packed_random(torch, m, k, 31)
+        sets = [(x, packed_random(torch, n, k, 40 + i), torch.empty((m, n), dtype=torch.int32, device="cuda"))
+                for i in range(nsets)]
+
+        def launch(t, m=m, n=n, k=k):
+            lib.gemm_s4s4s32(t[0], t[1], t[2], m, n, k)
+
+        ev_ms, _ = time_launches(torch, launch, sets, max(steps, 200), max(warmup, 20))
+        algo_bytes = m * k // 2 + n * k // 2 + 4 * m * n
+        gbs = algo_bytes / (ev_ms * 1e-3) / 1e9
+        out.append({"shape": [m, n, k], "kernel": lib.kernel_for_shape(m, n, k), "us_per_launch": ev_ms * 1e3,
+                    "bytes": algo_bytes, "GB/s": gbs, "frac_of_hbm_peak": gbs / HBM_PEAK_GBS})
+        del sets
+        torch.cuda.empty_cache()
+    return out
+
+
+def cpu_baseline(budget_s: float = 12.0):
+    """The oracle's loop nest (oracle_linear_ref_mt) on a row sample of the 8192^3
+    problem, all host threads the box grants us."""
+    from oracle import loader as oracle
+
+    threads = max(1, min(16, os.cpu_count() or 1))
+    rng = np.random.default_rng(7)
+    w = rng.integers(-8, 8, size=(N, K), dtype=np.int8).astype(np.int32)
+    # calibrate on one row per thread, then size the sample to the budget
+    rows = threads
+    x = rng.integers(-8, 8, size=(rows, K), dtype=np.int8).astype(np.int32)
+    t0 = time.perf_counter()
+    oracle.linear_ref(x, w, threads=threads)
+    dt = time.perf_counter() - t0
+    rows = int(max(threads, min(M, (budget_s / max(dt, 1e-3)) * rows)) // threads * threads)
+    x = rng.integers(-8, 8, size=(rows, K), dtype=np.int8).astype(np.int32)
+    t0 = time.perf_counter()
+    oracle.linear_ref(x, w, threads=threads)
+    dt = time.perf_counter() - t0
+    tops = 2.0 * rows * N * K / dt / 1e12
+    return {"value": tops, "unit": "TOPS", "cores": threads, "kind": "port",
+            "sample": f"{rows} of {M} rows of the 8192^3 problem (all {N} columns, full K), "
+                      f"{dt:.1f} s, oracle_linear_ref_mt with {threads} threads"}
+
+
+def measured_traffic():
+    """HBM bytes per launch of the GEMM kernel from rocprofv3 counter runs, if recorded."""
+    f = ROOT / "profiles" / "traffic.json"
+    if f.exists():
+        try:
+            return json.loads(f.read_text()).get("mfma_gemm_8192", {}).get("bytes_per_launch")
+        except Exception:
+            return None
+    return None
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-decode", action="store_true", help="skip the decode-shape leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only; run with --gpus 1 "
+              "(the path shards over N with no exchange step, see DESIGN.md)", file=sys.stderr)
+        return 2
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no HIP device visible", file=sys.stderr)
+        return 1
+    import int4linear_amd as lib
+
+    lib.init()
+    torch.cuda.set_device(0)
+
+    ev_ms, wall_ms = bench_gemm(torch, lib, args.steps, args.warmup)
+    ops = 2.0 * M * N * K
+    tops_kernel = ops / (ev_ms * 1e-3) / 1e12
+    tops_wall = ops / (wall_ms * 1e-3) / 1e12
+
+    result = {
+        "metric": "INT4 GEMM TOPS at M=N=K=8192 (% int8 MFMA peak); GB/s at M=16 decode",
+        "value": tops_wall,
+        "unit": "TOPS",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": wall_ms,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8",
+        "data": "synthetic",
+        "config": {"workload": "M=N=K=8192 s4*s4->s32 GEMM, uniform [-8,7], 3 rotating operand sets",
+                   "kernel": lib.kernel_for_shape(M, N, K), "M": M, "N": N, "K": K},
+        "pct_of_int8_mfma_peak": 100.0 * tops_wall / INT8_MFMA_PEAK_TOPS,
+        "roofline": {"bound": "mfma", "achieved": tops_kernel, "peak": INT8_MFMA_PEAK_TOPS,
+                     "unit": "TFLOP/s", "frac": tops_kernel / INT8_MFMA_PEAK_TOPS,
+                     "traffic": measured_traffic(),
+                     "note": "integer ops: 2*M*N*K per launch / mean launch time (HIP events)",
+                     "kernel_ms": ev_ms},
+    }
+    if not args.no_decode:
+        dec = bench_decode(torch, lib, args.steps, args.warmup)
+        result["decode"] = dec
+        big = [d for d in dec if d["shape"] != [16, 4096, 4096]]
+        result["decode_GB/s_M16"] = sum(d["GB/s"] for d in big) / len(big)
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,111 @@
+/*
+ * int4linear.h -- host API of the MI355X (gfx950) signed-int4 linear-layer GEMM.
+ *
+ *   C[M x N] (int32, row-major, ld = N)  =  A[M x K] (s4)  *  B[N x K]^T (s4)
+ *
+ * A and B are K-contiguous and packed two signed 4-bit values per byte, element e of
+ * a row in byte e/2, even e in the low nibble (the layout written by the reference's
+ * utils/packer.cpp:3-18).  Row stride is K/2 bytes.  Accumulation is exact int32.
+ *
+ * Two layers are exported by libint4linear.so:
+ *   1. a C ABI (extern "C", plain pointers and sizes, status codes, asynchronous on a
+ *      caller-supplied HIP stream) -- the drop-in boundary other languages bind to;
+ *   2. the reference's own C++-linkage entry points (linear_vN_launch, pack, unpack)
+ *      with the reference's signatures and blocking behaviour, implemented on top of 1.
+ *
+ * All pointers named *_d are device pointers owned by the caller.  The library makes
+ * no device allocation in any entry point declared here.
+ */
+#ifndef INT4LINEAR_H
+#define INT4LINEAR_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Status codes returned by every C-ABI entry point. */
+enum {
+    INT4LINEAR_OK = 0,
+    INT4LINEAR_ERR_SHAPE = 1,       /* negative dimension, or K not a multiple of 8      */
+    INT4LINEAR_ERR_NULL = 2,        /* null pointer with a non-empty operand             */
+    INT4LINEAR_ERR_ALIGN = 3,       /* operand base not 16-byte aligned                  */
+    INT4LINEAR_ERR_HIP = 4,         /* a HIP runtime call failed (see last_hip_error)    */
+    INT4LINEAR_ERR_UNSUPPORTED = 5, /* the requested kernel cannot run this shape        */
+    INT4LINEAR_ERR_NO_DEVICE = 6    /* no gfx950 device is visible                       */
+};
+
+/* Kernel selector for int4linear_gemm_s4s4s32_ex. */
+enum {
+    INT4LINEAR_KERNEL_AUTO = 0,   /* shape-based dispatch (what the plain entry uses)    */
+    INT4LINEAR_KERNEL_SIMPLE = 1, /* one thread per output, scalar nibble decode; any K%8==0 */
+    INT4LINEAR_KERNEL_MFMA = 2,   /* LDS-pipelined v_mfma_i32_16x16x64_i8 kernel; K%128==0 */
+    INT4LINEAR_KERNEL_SKINNY = 3  /* weight-streaming kernel for M <= 64; K%128==0       */
+};
+
+/* One-time set-up for the current HIP device (queries the CU count, raises the
+ * dynamic-LDS limit of the kernels).  Called implicitly by the other entry points;
+ * idempotent and thread-safe.  Replaces the per-call cudaFuncSetAttribute of
+ * kernels/linear_v21.cu:14-18. */
+int int4linear_init(void);
+
+/* The GEMM.  Asynchronous: work is enqueued on `stream` (a hipStream_t, NULL = the
+ * default stream) and the call returns without synchronising.  C is fully overwritten.
+ * M == 0 or N == 0 is a no-op; K == 0 zero-fills C.
+ * Replaces kernels/linear_v21.cu:9-49 (linear_v21_launch) minus its device-wide
+ * synchronisation, and the direct kernel launch of test/benchmark.cu:46-72. */
+int int4linear_gemm_s4s4s32(const void *a_packed_d, const void *b_packed_d, void *c_d,
+                            int m, int n, int k, void *stream);
+
+/* Same as above with an explicit kernel choice (INT4LINEAR_KERNEL_*).  Returns
+ * INT4LINEAR_ERR_UNSUPPORTED when that kernel cannot run the shape. */
+int int4linear_gemm_s4s4s32_ex(const void *a_packed_d, const void *b_packed_d, void *c_d,
+                               int m, int n, int k, int kernel, void *stream);
+
+/* Device-side counterparts of utils/packer.cpp:3-18 (pack) and :20-31 (unpack):
+ * src_d / dst_d are device arrays with the reference's host layouts (m x n ints
+ * unpacked, m x ceil(n/8) 32-bit words packed).  Asynchronous on `stream`. */
+int int4linear_pack_s32_to_s4(const int *src_d, int *dst_d, int m, int n, void *stream);
+int int4linear_unpack_s4_to_s32(const int *src_d, int *dst_d, int m, int n, void *stream);
+
+/* Name of the kernel INT4LINEAR_KERNEL_AUTO would pick for a shape ("simple", "mfma",
+ * "skinny"); never NULL. */
+const char *int4linear_kernel_for_shape(int m, int n, int k);
+
+/* Human-readable text for a status code; never NULL. */
+const char *int4linear_status_string(int status);
+
+/* hipError_t value of the most recent failing HIP call on this thread (0 if none). */
+int int4linear_last_hip_error(void);
+
+/* Number of compute units the library saw on the current device (0 before init). */
+int int4linear_device_cu_count(void);
+
+#ifdef __cplusplus
+} /* extern "C" */
+
+/*
+ * The reference's entry points, C++ linkage, same signatures and semantics:
+ * blocking (the call returns after the device has finished), default stream, void
+ * return, silent on success.  All seven names run the same dispatch; v0 always takes
+ * the simple kernel so it can serve as an independent on-device cross-check.
+ *   kernels/linear_v0.h:168   kernels/linear_v1.h:208   kernels/linear_v2.h:284
+ *   kernels/linear_v10.h:492  kernels/linear_v11.h:658  kernels/linear_v20.h:738
+ *   kernels/linear_v21.h:760
+ * A failing call prints one line to stderr (the reference prints only under __DEBUG,
+ * kernels/linear_v21.cu:41-47).
+ */
+void linear_v0_launch(void *x_packed_d, void *w_packed_d, void *y_d, int m, int n, int k);
+void linear_v1_launch(void *x_packed_d, void *w_packed_d, void *y_d, int m, int n, int k);
+void linear_v2_launch(void *x_packed_d, void *w_packed_d, void *y_d, int m, int n, int k);
+void linear_v10_launch(void *x_packed_d, void *w_packed_d, void *y_d, int m, int n, int k);
+void linear_v11_launch(void *x_packed_d, void *w_packed_d, void *y_d, int m, int n, int k);
+void linear_v20_launch(void *x_packed_d, void *w_packed_d, void *y_d, int m, int n, int k);
+void linear_v21_launch(void *x_packed_d, void *w_packed_d, void *y_d, int m, int n, int k);
+
+/* Host packer with the reference's signatures (utils/packer.h:5-6): host arrays in,
+ * host arrays out. */
+void pack(const int *src, int *dst, const int m, const int n);
+void unpack(const int *src, int *dst, const int m, const int n);
+#endif
+
+#endif /* INT4LINEAR_H */

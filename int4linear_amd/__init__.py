@@ -1,0 +1,24 @@
+"""MI355X (gfx950) signed-int4 linear-layer GEMM behind the Int4Linear host API.
+
+The compute lives in ``lib/libint4linear.so`` (HIP kernels + C ABI, declared in
+``include/int4linear.h``); this package is the thin host-side mirror of the reference's
+``linear_vN_launch`` / ``pack`` / ``unpack`` interface.
+"""
+from .api import (  # noqa: F401
+    gemm_s4s4s32,
+    init,
+    kernel_for_shape,
+    linear_v0_launch,
+    linear_v1_launch,
+    linear_v2_launch,
+    linear_v10_launch,
+    linear_v11_launch,
+    linear_v20_launch,
+    linear_v21_launch,
+    pack,
+    pack_device,
+    pack_rows,
+    unpack,
+    unpack_device,
+)
+from ._lib import Int4LinearError  # noqa: F401

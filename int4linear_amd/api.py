@@ -1,0 +1,132 @@
+"""Host-side mirror of the reference's interface, on top of the C ABI.
+
+Names and argument meaning follow the reference:
+  linear_vN_launch(x_packed_d, w_packed_d, y_d, m, n, k)   kernels/linear_v21.h:760 (and v0..v20)
+  pack(src, dst, m, n) / unpack(src, dst, m, n)            utils/packer.h:5-6
+Device operands are torch tensors on a ROCm device (torch is only the owner of the
+device memory and the stream) or raw integer device addresses.
+"""
+from __future__ import annotations
+
+import ctypes
+
+import numpy as np
+
+from . import _lib
+
+KERNELS = {"auto": 0, "simple": 1, "mfma": 2, "skinny": 3}
+
+
+def _ptr(obj) -> int:
+    """Device (or host) address of a torch tensor / numpy array / raw int."""
+    if obj is None:
+        return 0
+    if isinstance(obj, int):
+        return obj
+    if isinstance(obj, np.ndarray):
+        return obj.ctypes.data
+    return obj.data_ptr()  # torch.Tensor
+
+
+def _current_stream() -> int:
+    import torch
+
+    return torch.cuda.current_stream().cuda_stream
+
+
+def init() -> None:
+    """One-time device set-up (idempotent)."""
+    lib = _lib.load()
+    _lib.check(lib.int4linear_init())
+
+
+def gemm_s4s4s32(a_packed_d, b_packed_d, c_d, m: int, n: int, k: int, *, kernel: str = "auto",
+                 stream: int | None = None) -> None:
+    """Asynchronous C = A * B^T on `stream` (default: torch's current stream)."""
+    lib = _lib.load()
+    if stream is None:
+        stream = _current_stream()
+    st = lib.int4linear_gemm_s4s4s32_ex(_ptr(a_packed_d), _ptr(b_packed_d), _ptr(c_d), m, n, k,
+                                        KERNELS[kernel], ctypes.c_void_p(stream))
+    _lib.check(st)
+
+
+def kernel_for_shape(m: int, n: int, k: int) -> str:
+    return _lib.load().int4linear_kernel_for_shape(m, n, k).decode()
+
+
+def pack_device(src_d, dst_d, m: int, n: int, *, stream: int | None = None) -> None:
+    lib = _lib.load()
+    if stream is None:
+        stream = _current_stream()
+    _lib.check(lib.int4linear_pack_s32_to_s4(_ptr(src_d), _ptr(dst_d), m, n, ctypes.c_void_p(stream)))
+
+
+def unpack_device(src_d, dst_d, m: int, n: int, *, stream: int | None = None) -> None:
+    lib = _lib.load()
+    if stream is None:
+        stream = _current_stream()
+    _lib.check(lib.int4linear_unpack_s4_to_s32(_ptr(src_d), _ptr(dst_d), m, n, ctypes.c_void_p(stream)))
+
+
+def _launch(symbol: str, x_packed_d, w_packed_d, y_d, m: int, n: int, k: int) -> None:
+    lib = _lib.load()
+    getattr(lib, symbol)(_ptr(x_packed_d), _ptr(w_packed_d), _ptr(y_d), m, n, k)
+
+
+# Blocking entry points with the reference's names: default stream, device-synchronised
+# on return, no status (a failure prints one line to stderr).
+def linear_v0_launch(x_packed_d, w_packed_d, y_d, m, n, k):
+    _launch("_Z16linear_v0_launchPvS_S_iii", x_packed_d, w_packed_d, y_d, m, n, k)
+
+
+def linear_v1_launch(x_packed_d, w_packed_d, y_d, m, n, k):
+    _launch("_Z16linear_v1_launchPvS_S_iii", x_packed_d, w_packed_d, y_d, m, n, k)
+
+
+def linear_v2_launch(x_packed_d, w_packed_d, y_d, m, n, k):
+    _launch("_Z16linear_v2_launchPvS_S_iii", x_packed_d, w_packed_d, y_d, m, n, k)
+
+
+def linear_v10_launch(x_packed_d, w_packed_d, y_d, m, n, k):
+    _launch("_Z17linear_v10_launchPvS_S_iii", x_packed_d, w_packed_d, y_d, m, n, k)
+
+
+def linear_v11_launch(x_packed_d, w_packed_d, y_d, m, n, k):
+    _launch("_Z17linear_v11_launchPvS_S_iii", x_packed_d, w_packed_d, y_d, m, n, k)
+
+
+def linear_v20_launch(x_packed_d, w_packed_d, y_d, m, n, k):
+    _launch("_Z17linear_v20_launchPvS_S_iii", x_packed_d, w_packed_d, y_d, m, n, k)
+
+
+def linear_v21_launch(x_packed_d, w_packed_d, y_d, m, n, k):
+    _launch("_Z17linear_v21_launchPvS_S_iii", x_packed_d, w_packed_d, y_d, m, n, k)
+
+
+def pack(src: np.ndarray, dst: np.ndarray, m: int, n: int) -> None:
+    """Host packer: src is m*n int32 values, dst receives m*ceil(n/8) int32 words."""
+    lib = _lib.load()
+    assert src.dtype == np.int32 and dst.dtype == np.int32
+    assert src.flags.c_contiguous and dst.flags.c_contiguous
+    assert src.size >= m * n and dst.size >= m * ((n + 7) // 8)
+    lib._Z4packPKiPiii(_ptr(src), _ptr(dst), m, n)
+
+
+def unpack(src: np.ndarray, dst: np.ndarray, m: int, n: int) -> None:
+    """Host unpacker: inverse of pack."""
+    lib = _lib.load()
+    assert src.dtype == np.int32 and dst.dtype == np.int32
+    assert src.flags.c_contiguous and dst.flags.c_contiguous
+    assert src.size >= m * ((n + 7) // 8) and dst.size >= m * n
+    lib._Z6unpackPKiPiii(_ptr(src), _ptr(dst), m, n)
+
+
+def pack_rows(values: np.ndarray) -> np.ndarray:
+    """Convenience: pack a 2-D integer array (any int dtype, values in [-8, 7]) into the
+    m x ceil(n/8) int32 word layout."""
+    m, n = values.shape
+    src = np.ascontiguousarray(values, dtype=np.int32)
+    dst = np.empty((m, (n + 7) // 8), dtype=np.int32)
+    pack(src, dst, m, n)
+    return dst

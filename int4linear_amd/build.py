@@ -1,0 +1,84 @@
+"""Builds libint4linear.so (HIP kernels + C ABI) for gfx950 with hipcc, in-tree.
+
+Run as ``python -m int4linear_amd.build``.  hipcc cross-compiles for gfx950 without a
+GPU, so this works on a CPU-only machine.  The library lands in
+``int4linear_amd/lib/libint4linear.so``.
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+PKG_DIR = Path(__file__).resolve().parent
+CSRC = PKG_DIR / "csrc"
+LIB_DIR = PKG_DIR / "lib"
+OBJ_DIR = PKG_DIR / "csrc" / "build"
+LIB_PATH = LIB_DIR / "libint4linear.so"
+
+HIP_SOURCES = ["api.hip", "kernels_simple.hip", "kernels_mfma.hip", "kernels_skinny.hip"]
+CXX_SOURCES = ["packer_host.cpp"]
+
+# Packed-FP32 VALU forms are switched off for every device compile of this project.
+HIP_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def _hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found; ROCm is required to build int4linear_amd")
+    return exe
+
+
+def _run(cmd: list[str]) -> None:
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("command failed: " + " ".join(cmd) + "\n" + proc.stdout)
+    # hipcc's host pass warns that it does not know the packed-fp32 feature: harmless.
+    noise = ("is not a recognized feature", "warning generated", "warnings generated")
+    out = "\n".join(l for l in proc.stdout.splitlines() if l and not any(n in l for n in noise))
+    if out.strip():
+        sys.stderr.write(out + "\n")
+
+
+def build_library(verbose: bool = False, save_temps: bool = False) -> Path:
+    """Compile every source and link the shared library.  Always recompiles."""
+    hipcc = _hipcc()
+    LIB_DIR.mkdir(exist_ok=True)
+    OBJ_DIR.mkdir(exist_ok=True)
+    jobs = []
+    for src in HIP_SOURCES:
+        obj = OBJ_DIR / (src + ".o")
+        cmd = [hipcc, *HIP_FLAGS, "-c", str(CSRC / src), "-o", str(obj)]
+        if save_temps:
+            cmd.insert(1, "-save-temps=obj")
+        jobs.append((cmd, obj))
+    for src in CXX_SOURCES:
+        obj = OBJ_DIR / (src + ".o")
+        jobs.append(([hipcc, "-O3", "-std=c++17", "-fPIC", "-c", str(CSRC / src), "-o", str(obj)], obj))
+    if verbose:
+        for cmd, _ in jobs:
+            print(" ".join(cmd))
+    with ThreadPoolExecutor(max_workers=min(8, len(jobs))) as pool:
+        list(pool.map(lambda j: _run(j[0]), jobs))
+    link = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(LIB_PATH)]
+    link += [str(obj) for _, obj in jobs]
+    if verbose:
+        print(" ".join(link))
+    _run(link)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    path = build_library(verbose="-v" in sys.argv, save_temps="--save-temps" in sys.argv)
+    print(path)

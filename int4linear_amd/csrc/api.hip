@@ -1,0 +1,270 @@
+// C ABI of libint4linear.so, shape dispatch, and the reference's C++-linkage shims.
+#include "../../include/int4linear.h"
+#include "kernels.h"
+
+#include <cstdint>
+#include <cstdio>
+#include <mutex>
+
+namespace {
+
+using namespace int4linear;
+
+constexpr int kMaxDevices = 64;
+
+struct PerDevice {
+    std::once_flag once;
+    hipError_t init_error = hipSuccess;
+    int status = INT4LINEAR_OK;
+    DeviceInfo info;
+};
+
+PerDevice g_devices[kMaxDevices];
+thread_local int t_last_hip_error = 0;
+
+int fail_hip(hipError_t e)
+{
+    t_last_hip_error = (int)e;
+    return INT4LINEAR_ERR_HIP;
+}
+
+// Set-up for the device that is current on the calling thread; returns its record.
+int ensure_init(PerDevice **out)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) {
+        t_last_hip_error = (int)e;
+        return INT4LINEAR_ERR_NO_DEVICE;
+    }
+    if (dev < 0 || dev >= kMaxDevices)
+        return INT4LINEAR_ERR_NO_DEVICE;
+    PerDevice &pd = g_devices[dev];
+    std::call_once(pd.once, [&pd, dev]() {
+        hipDeviceProp_t prop;
+        hipError_t err = hipGetDeviceProperties(&prop, dev);
+        if (err != hipSuccess) {
+            pd.init_error = err;
+            pd.status = INT4LINEAR_ERR_HIP;
+            return;
+        }
+        pd.info.cu_count = prop.multiProcessorCount;
+        pd.info.lds_per_cu = (int)prop.maxSharedMemoryPerMultiProcessor;
+        err = mfma_init(pd.info);
+        if (err != hipSuccess) {
+            pd.init_error = err;
+            pd.status = INT4LINEAR_ERR_HIP;
+        }
+    });
+    if (pd.status != INT4LINEAR_OK) {
+        t_last_hip_error = (int)pd.init_error;
+        return pd.status;
+    }
+    if (out)
+        *out = &pd;
+    return INT4LINEAR_OK;
+}
+
+bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
+
+int pick_kernel(int m, int n, int k)
+{
+    if (skinny_supports(m, n, k))
+        return INT4LINEAR_KERNEL_SKINNY;
+    if (mfma_supports(m, n, k))
+        return INT4LINEAR_KERNEL_MFMA;
+    return INT4LINEAR_KERNEL_SIMPLE;
+}
+
+int gemm_impl(const void *a, const void *b, void *c, int m, int n, int k, int kernel,
+              void *stream_v)
+{
+    if (m < 0 || n < 0 || k < 0 || (k % 8) != 0)
+        return INT4LINEAR_ERR_SHAPE;
+    if (kernel < INT4LINEAR_KERNEL_AUTO || kernel > INT4LINEAR_KERNEL_SKINNY)
+        return INT4LINEAR_ERR_UNSUPPORTED;
+    if (m == 0 || n == 0)
+        return INT4LINEAR_OK;
+    if (!c)
+        return INT4LINEAR_ERR_NULL;
+    if (k > 0 && (!a || !b))
+        return INT4LINEAR_ERR_NULL;
+    if (!aligned16(c) || (k > 0 && (!aligned16(a) || !aligned16(b))))
+        return INT4LINEAR_ERR_ALIGN;
+
+    PerDevice *pd = nullptr;
+    int st = ensure_init(&pd);
+    if (st != INT4LINEAR_OK)
+        return st;
+    hipStream_t stream = (hipStream_t)stream_v;
+
+    if (k == 0) {
+        hipError_t e = launch_zero_i32((int *)c, (size_t)m * (size_t)n, stream);
+        return e == hipSuccess ? INT4LINEAR_OK : fail_hip(e);
+    }
+
+    if (kernel == INT4LINEAR_KERNEL_AUTO)
+        kernel = pick_kernel(m, n, k);
+
+    hipError_t e = hipSuccess;
+    switch (kernel) {
+    case INT4LINEAR_KERNEL_SIMPLE:
+        e = launch_simple(a, b, c, m, n, k, stream);
+        break;
+    case INT4LINEAR_KERNEL_MFMA:
+        if (!mfma_supports(m, n, k))
+            return INT4LINEAR_ERR_UNSUPPORTED;
+        e = launch_mfma(a, b, c, m, n, k, pd->info, stream);
+        break;
+    case INT4LINEAR_KERNEL_SKINNY:
+        if (!skinny_supports(m, n, k))
+            return INT4LINEAR_ERR_UNSUPPORTED;
+        e = launch_skinny(a, b, c, m, n, k, pd->info, stream);
+        break;
+    default:
+        return INT4LINEAR_ERR_UNSUPPORTED;
+    }
+    return e == hipSuccess ? INT4LINEAR_OK : fail_hip(e);
+}
+
+// Blocking call in the reference's style: enqueue on the default stream, then wait for
+// the device, as kernels/linear_v21.cu:37-39 does.
+void launch_blocking(const char *name, void *x, void *w, void *y, int m, int n, int k, int kernel)
+{
+    int st = gemm_impl(x, w, y, m, n, k, kernel, nullptr);
+    if (st == INT4LINEAR_OK) {
+        hipError_t e = hipDeviceSynchronize();
+        if (e != hipSuccess)
+            st = fail_hip(e);
+    }
+    if (st != INT4LINEAR_OK)
+        std::fprintf(stderr, "%s FAILED: %s (hip error %d)\n", name, int4linear_status_string(st),
+                     t_last_hip_error);
+}
+
+}  // namespace
+
+extern "C" {
+
+int int4linear_init(void) { return ensure_init(nullptr); }
+
+int int4linear_gemm_s4s4s32(const void *a_packed_d, const void *b_packed_d, void *c_d, int m,
+                            int n, int k, void *stream)
+{
+    return gemm_impl(a_packed_d, b_packed_d, c_d, m, n, k, INT4LINEAR_KERNEL_AUTO, stream);
+}
+
+int int4linear_gemm_s4s4s32_ex(const void *a_packed_d, const void *b_packed_d, void *c_d, int m,
+                               int n, int k, int kernel, void *stream)
+{
+    return gemm_impl(a_packed_d, b_packed_d, c_d, m, n, k, kernel, stream);
+}
+
+int int4linear_pack_s32_to_s4(const int *src_d, int *dst_d, int m, int n, void *stream)
+{
+    if (m < 0 || n < 0)
+        return INT4LINEAR_ERR_SHAPE;
+    if (m == 0 || n == 0)
+        return INT4LINEAR_OK;
+    if (!src_d || !dst_d)
+        return INT4LINEAR_ERR_NULL;
+    int st = ensure_init(nullptr);
+    if (st != INT4LINEAR_OK)
+        return st;
+    hipError_t e = launch_pack(src_d, dst_d, m, n, (hipStream_t)stream);
+    return e == hipSuccess ? INT4LINEAR_OK : fail_hip(e);
+}
+
+int int4linear_unpack_s4_to_s32(const int *src_d, int *dst_d, int m, int n, void *stream)
+{
+    if (m < 0 || n < 0)
+        return INT4LINEAR_ERR_SHAPE;
+    if (m == 0 || n == 0)
+        return INT4LINEAR_OK;
+    if (!src_d || !dst_d)
+        return INT4LINEAR_ERR_NULL;
+    int st = ensure_init(nullptr);
+    if (st != INT4LINEAR_OK)
+        return st;
+    hipError_t e = launch_unpack(src_d, dst_d, m, n, (hipStream_t)stream);
+    return e == hipSuccess ? INT4LINEAR_OK : fail_hip(e);
+}
+
+const char *int4linear_kernel_for_shape(int m, int n, int k)
+{
+    if (m < 0 || n < 0 || k < 0 || (k % 8) != 0)
+        return "invalid";
+    switch (pick_kernel(m, n, k)) {
+    case INT4LINEAR_KERNEL_SKINNY:
+        return "skinny";
+    case INT4LINEAR_KERNEL_MFMA:
+        return "mfma";
+    default:
+        return "simple";
+    }
+}
+
+const char *int4linear_status_string(int status)
+{
+    switch (status) {
+    case INT4LINEAR_OK:
+        return "ok";
+    case INT4LINEAR_ERR_SHAPE:
+        return "invalid shape (negative dimension or K not a multiple of 8)";
+    case INT4LINEAR_ERR_NULL:
+        return "null pointer for a non-empty operand";
+    case INT4LINEAR_ERR_ALIGN:
+        return "operand base pointer is not 16-byte aligned";
+    case INT4LINEAR_ERR_HIP:
+        return "HIP runtime error";
+    case INT4LINEAR_ERR_UNSUPPORTED:
+        return "requested kernel does not support this shape";
+    case INT4LINEAR_ERR_NO_DEVICE:
+        return "no usable HIP device";
+    default:
+        return "unknown status";
+    }
+}
+
+int int4linear_last_hip_error(void) { return t_last_hip_error; }
+
+int int4linear_device_cu_count(void)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+        return 0;
+    return g_devices[dev].info.cu_count;
+}
+
+}  // extern "C"
+
+// ---- the reference's C++-linkage entry points ------------------------------------------
+
+void linear_v0_launch(void *x, void *w, void *y, int m, int n, int k)
+{
+    launch_blocking("linear_v0_launch", x, w, y, m, n, k, INT4LINEAR_KERNEL_SIMPLE);
+}
+void linear_v1_launch(void *x, void *w, void *y, int m, int n, int k)
+{
+    launch_blocking("linear_v1_launch", x, w, y, m, n, k, INT4LINEAR_KERNEL_AUTO);
+}
+void linear_v2_launch(void *x, void *w, void *y, int m, int n, int k)
+{
+    launch_blocking("linear_v2_launch", x, w, y, m, n, k, INT4LINEAR_KERNEL_AUTO);
+}
+void linear_v10_launch(void *x, void *w, void *y, int m, int n, int k)
+{
+    launch_blocking("linear_v10_launch", x, w, y, m, n, k, INT4LINEAR_KERNEL_AUTO);
+}
+void linear_v11_launch(void *x, void *w, void *y, int m, int n, int k)
+{
+    launch_blocking("linear_v11_launch", x, w, y, m, n, k, INT4LINEAR_KERNEL_AUTO);
+}
+void linear_v20_launch(void *x, void *w, void *y, int m, int n, int k)
+{
+    launch_blocking("linear_v20_launch", x, w, y, m, n, k, INT4LINEAR_KERNEL_AUTO);
+}
+void linear_v21_launch(void *x, void *w, void *y, int m, int n, int k)
+{
+    launch_blocking("linear_v21_launch", x, w, y, m, n, k, INT4LINEAR_KERNEL_AUTO);
+}

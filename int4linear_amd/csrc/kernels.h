@@ -1,0 +1,36 @@
+// Internal launcher interface between the C ABI (api.hip) and the kernel files.
+// Every launcher enqueues on `stream` and returns the hipError_t of the launch.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace int4linear {
+
+struct DeviceInfo {
+    int cu_count = 0;      // compute units on the device
+    int lds_per_cu = 0;    // bytes of LDS a workgroup may use
+};
+
+// One thread per output, scalar nibble decode.  Any M, N >= 1 and K % 8 == 0.
+hipError_t launch_simple(const void *a, const void *b, void *c, int m, int n, int k,
+                         hipStream_t stream);
+
+// LDS-pipelined MFMA kernel.  Requires K % 128 == 0, K >= 128.
+bool mfma_supports(int m, int n, int k);
+hipError_t mfma_init(const DeviceInfo &dev);
+hipError_t launch_mfma(const void *a, const void *b, void *c, int m, int n, int k,
+                       const DeviceInfo &dev, hipStream_t stream);
+
+// Weight-streaming kernel for skinny M.  Requires M <= 64, K % 128 == 0.
+bool skinny_supports(int m, int n, int k);
+hipError_t launch_skinny(const void *a, const void *b, void *c, int m, int n, int k,
+                         const DeviceInfo &dev, hipStream_t stream);
+
+// Device packer / unpacker, utils/packer.cpp layouts.
+hipError_t launch_pack(const int *src, int *dst, int m, int n, hipStream_t stream);
+hipError_t launch_unpack(const int *src, int *dst, int m, int n, hipStream_t stream);
+
+// Fill `count` int32 words with zero (a kernel, so callers may capture it in a graph).
+hipError_t launch_zero_i32(int *dst, size_t count, hipStream_t stream);
+
+}  // namespace int4linear

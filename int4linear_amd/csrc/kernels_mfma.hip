@@ -1,0 +1,383 @@
+// LDS-pipelined int8-MFMA GEMM over packed signed-int4 operands for gfx950 (CDNA4).
+//
+// gfx950 has no 4-bit integer MFMA, so nibbles are widened to int8 in registers and fed
+// to v_mfma_i32_16x16x64_i8.  The widening keeps each nibble in the HIGH half of its
+// byte: for a packed word w,  (w << 4) & 0xF0F0F0F0  holds the even-k nibbles and
+// w & 0xF0F0F0F0 the odd-k nibbles, each as the signed byte 16*value (the nibble's own
+// sign bit lands in bit 7, so no sign-extension step exists).  Both operands carry the
+// factor 16, every product carries 256, and C = acc >> 8 exactly.  |acc| <= K * 2^14, so
+// int32 holds it for K <= 131071; the launcher refuses larger K.
+//
+// A dot product does not care in which order k is visited as long as both operands
+// visit it in the same order, so even and odd nibbles are never re-interleaved and a
+// lane simply owns whatever 32 nibbles its 16-byte LDS read returns.
+//
+// Data movement per workgroup (tile BM x BN of C, K consumed 128 nibbles per stage):
+//   HBM/L2 --global_load_lds_dwordx4 (16 B per lane, straight into LDS)--> NSTAGE-deep ring
+//   LDS    --ds_read_b128 (bank-conflict-free through a 16-byte-chunk XOR swizzle)--> VGPRs
+//   VGPRs  --3 VALU ops per packed dword--> int8 operands --MFMA--> int32 accumulators
+//   accumulators --buffer_store_dwordx4 (W is the MFMA A operand, so a lane's four
+//                 accumulators are four consecutive n)--> C
+// The kernel is persistent: gridDim.x workgroups walk a list of tiles, and the load
+// ring runs NSTAGE-1 stages ahead of the math ACROSS tile boundaries, so the next
+// tile's first stages are in flight while the current tile stores C.
+#include "kernels.h"
+
+namespace int4linear {
+
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+
+#define I4L_LDS(p) ((__attribute__((address_space(3))) void *)(p))
+
+// s_waitcnt immediate for gfx9: vmcnt[3:0] in bits 3:0, vmcnt[5:4] in bits 15:14,
+// expcnt (bits 6:4) and lgkmcnt (bits 11:8) left at "no wait".
+#define I4L_VMCNT(n) ((0x0F70) | ((n) & 0xF) | ((((n) >> 4) & 0x3) << 14))
+
+// 16 bytes per lane from global memory straight into LDS: lane l's data lands at LDS
+// byte lds_addr + 16*l.  Global address = wave-uniform base (SGPR pair) + per-lane
+// 32-bit offset.  M0 carries the LDS address; one wait state separates its write from
+// the load that reads it.  The compiler does not count this load in its own vmcnt
+// bookkeeping, which only makes the waits it inserts for its own accesses stricter.
+__device__ __forceinline__ void dma16(const void *sbase, unsigned voff, unsigned lds_addr)
+{
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(voff), "s"(sbase), "s"(lds_addr)
+                 : "memory");
+}
+
+// Hides a value's origin from the optimiser so that work derived from it stays where
+// it is written instead of being hoisted out of the stage loop into live registers.
+__device__ __forceinline__ int opaque(int v)
+{
+    asm volatile("" : "+v"(v));
+    return v;
+}
+
+constexpr int kStageK = 128;                 // nibbles of K per pipeline stage
+constexpr int kRowBytes = kStageK / 2;       // bytes per LDS row (64)
+constexpr int kChunkRows = 16;               // rows moved by one 64-lane 16-byte load
+constexpr int kChunkBytes = kChunkRows * kRowBytes;  // 1 KiB
+
+// Tile configuration.  A workgroup is WAVES_M x WAVES_N wavefronts; each owns
+// FM x FN MFMA tiles of 16x16, i.e. a (FM*16) x (FN*16) patch of C.
+template <int WAVES_M_, int WAVES_N_, int FM_, int FN_, int NSTAGE_, int OCC_>
+struct TileConfig {
+    static constexpr int WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
+    static constexpr int FM = FM_, FN = FN_;
+    static constexpr int NSTAGE = NSTAGE_;
+    static constexpr int OCC = OCC_;  // workgroups per CU the register budget allows
+    static constexpr int NWAVES = WAVES_M * WAVES_N;
+    static constexpr int THREADS = NWAVES * 64;
+    static constexpr int BM = WAVES_M * FM * 16;
+    static constexpr int BN = WAVES_N * FN * 16;
+    static constexpr int X_CHUNKS = BM / kChunkRows;
+    static constexpr int W_CHUNKS = BN / kChunkRows;
+    static constexpr int CH = (X_CHUNKS + W_CHUNKS) / NWAVES;  // loads per wave per stage
+    static constexpr int X_CH = X_CHUNKS / NWAVES;             // of which from X
+    static constexpr int STAGE_BYTES = (BM + BN) * kRowBytes;
+    static constexpr int LDS_BYTES = STAGE_BYTES * NSTAGE;
+    static constexpr int STORES = FM * FN;  // dwordx4 stores per lane per tile
+    static_assert(X_CHUNKS % NWAVES == 0 && W_CHUNKS % NWAVES == 0, "chunks must split evenly");
+    static_assert((NSTAGE - 2) * CH <= 63, "vmcnt is six bits");
+};
+
+// Which 16-byte slot of its 64-byte LDS row holds logical chunk g of row r:  g ^ swz(r).
+// With rows 64 B apart, sixteen lanes reading the same g of rows 0..15 touch sixteen
+// different 16-byte bank groups of a 256-byte window, and any eight consecutive of them
+// touch eight different groups of a 128-byte window.
+__device__ __forceinline__ int swz(int r) { return ((r >> 1) + (r >> 3)) & 3; }
+
+// Tile order.  Workgroup ids go round-robin over the 8 XCDs, each with a private L2, so
+// the tiles that run together on one XCD (ids congruent mod 8, consecutive quotients)
+// are given consecutive positions of a grouped order: 8 tile-rows tall, column-major
+// inside the group.  32 consecutive positions are then an 8x4 patch sharing rows of A
+// and B in that L2.
+__device__ __forceinline__ void tile_coords(int v, int total, int tiles_m, int tiles_n,
+                                            int &tm, int &tn)
+{
+    constexpr int kXcd = 8, kGroup = 8;
+    const int x = v % kXcd, j = v / kXcd;
+    const int cnt = total / kXcd, rem = total % kXcd;
+    const int q = x * cnt + (x < rem ? x : rem) + j;
+    const int per_group = kGroup * tiles_n;
+    const int group = q / per_group;
+    const int first_m = group * kGroup;
+    const int gsz = (tiles_m - first_m < kGroup) ? (tiles_m - first_m) : kGroup;
+    const int in_group = q % per_group;
+    tm = first_m + in_group % gsz;
+    tn = in_group / gsz;
+}
+
+template <class C, bool VEC_STORE>
+__global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
+    const uint8_t *__restrict__ X, const uint8_t *__restrict__ W, int32_t *__restrict__ Y,
+    int M, int N, int K, int tiles_m, int tiles_n)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wm = wave / C::WAVES_N;
+    const int wn = wave % C::WAVES_N;
+    const int rowbytes = K >> 1;
+    const int KT = K / kStageK;
+    const int total_tiles = tiles_m * tiles_n;
+    const int nblk = gridDim.x;
+    const int bid = blockIdx.x;
+    if (bid >= total_tiles)
+        return;
+    const int my_tiles = (total_tiles - bid + nblk - 1) / nblk;
+    const int total_stages = my_tiles * KT;
+
+    // ---- load side -------------------------------------------------------------------
+    // Lane p of a chunk lands at LDS byte p*16 of that chunk: row p/4, slot p%4.
+    const int ld_row = lane >> 2;
+    const int ld_g = (lane & 3) ^ swz(ld_row);
+    unsigned voff[C::CH];            // per-chunk byte offset of this lane from the tile base
+    const uint8_t *xptr = X, *wptr = W;  // wave-uniform: tile base + k offset
+    int ld_it = 0, ld_k = 0, issued = 0;
+
+    const unsigned lds_base = (unsigned)(size_t)I4L_LDS(lds);
+
+    auto ld_setup_tile = [&](int it) {
+        int tm, tn;
+        tile_coords(bid + it * nblk, total_tiles, tiles_m, tiles_n, tm, tn);
+        const int m0 = tm * C::BM, n0 = tn * C::BN;
+        const int row = opaque(ld_row);
+#pragma unroll
+        for (int c = 0; c < C::CH; ++c) {
+            const bool is_x = c < C::X_CH;
+            const int ci = (is_x ? c : c - C::X_CH) * C::NWAVES + wave;
+            const int r = ci * kChunkRows + row;
+            const int lim = is_x ? (M - 1 - m0) : (N - 1 - n0);  // last valid row, tile-relative
+            const int rc = r < lim ? r : lim;
+            voff[c] = (unsigned)rc * (unsigned)rowbytes + (unsigned)ld_g * 16u;
+        }
+        xptr = X + (size_t)m0 * rowbytes;
+        wptr = W + (size_t)n0 * rowbytes;
+    };
+
+    auto ld_issue = [&]() {
+        const int buf = issued % C::NSTAGE;
+        const unsigned dst = lds_base + buf * C::STAGE_BYTES;
+#pragma unroll
+        for (int c = 0; c < C::CH; ++c) {
+            const bool is_x = c < C::X_CH;
+            const int ci = (is_x ? c : c - C::X_CH) * C::NWAVES + wave;
+            dma16(is_x ? xptr : wptr, voff[c],
+                  dst + (is_x ? 0 : C::BM * kRowBytes) + ci * kChunkBytes);
+        }
+        ++issued;
+        ++ld_k;
+        xptr += kRowBytes;
+        wptr += kRowBytes;
+        if (ld_k == KT) {
+            ld_k = 0;
+            ++ld_it;
+            if (ld_it < my_tiles)
+                ld_setup_tile(ld_it);
+        }
+    };
+
+    ld_setup_tile(0);
+#pragma unroll 1
+    for (int s = 0; s < C::NSTAGE - 1; ++s)
+        if (issued < total_stages)
+            ld_issue();
+
+    // ---- math side -------------------------------------------------------------------
+    // Lane l of a 16x16x64 MFMA supplies row l%16, k-chunk l/16 of both operands.
+    const int fr = lane & 15;
+    const int fg = lane >> 4;
+    const unsigned rd_off = (unsigned)fr * kRowBytes + (unsigned)((fg ^ swz(fr)) * 16);
+    const unsigned x_rd = rd_off + (unsigned)(wm * C::FM * 16 * kRowBytes);
+    const unsigned w_rd = rd_off + (unsigned)(C::BM * kRowBytes + wn * C::FN * 16 * kRowBytes);
+    const int himask = (int)0xF0F0F0F0u;
+
+    v4i acc[C::FN][C::FM];
+    int cur_it = 0, kk = 0;
+
+#pragma unroll 1
+    for (int gs = 0; gs < total_stages; ++gs) {
+        // Wait until this wave's loads of stage gs have landed.  Outstanding VMEM ops
+        // complete in order; `ahead` stages were issued after stage gs, and the C stores
+        // of the previous tile sit behind the loads of that tile's successor stages.
+        const int ahead = issued - 1 - gs;
+        if (ahead >= C::NSTAGE - 2) {
+            if (cur_it > 0 && kk < C::NSTAGE - 1) {
+                constexpr int with_stores = (C::NSTAGE - 2) * C::CH + (VEC_STORE ? C::STORES : 64);
+                __builtin_amdgcn_s_waitcnt(I4L_VMCNT(with_stores < 63 ? with_stores : 63));
+            } else {
+                __builtin_amdgcn_s_waitcnt(I4L_VMCNT((C::NSTAGE - 2) * C::CH));
+            }
+        } else {
+            __builtin_amdgcn_s_waitcnt(I4L_VMCNT(0));
+        }
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+
+        // Refill the buffer every wave finished reading before the barrier.
+        if (issued < total_stages)
+            ld_issue();
+
+        if (kk == 0) {
+#pragma unroll
+            for (int i = 0; i < C::FN; ++i)
+#pragma unroll
+                for (int j = 0; j < C::FM; ++j)
+                    acc[i][j] = (v4i){0, 0, 0, 0};
+        }
+
+        const uint8_t *stage = lds + (gs % C::NSTAGE) * C::STAGE_BYTES;
+        // W fragments are widened once per stage and stay live; X fragments stream
+        // through one at a time, which bounds the operand registers next to the
+        // FM*FN*4 accumulators.
+        v4i wlo[C::FN], whi[C::FN];
+#pragma unroll
+        for (int i = 0; i < C::FN; ++i) {
+            const v4i ww = *(const v4i *)(stage + w_rd + i * 16 * kRowBytes);
+            wlo[i] = (ww << 4) & himask;  // even-k nibbles
+            whi[i] = ww & himask;         // odd-k nibbles
+        }
+#pragma unroll
+        for (int j = 0; j < C::FM; ++j) {
+            const v4i xw = *(const v4i *)(stage + x_rd + j * 16 * kRowBytes);
+            const v4i xlo = (xw << 4) & himask;
+            const v4i xhi = xw & himask;
+#pragma unroll
+            for (int i = 0; i < C::FN; ++i) {
+                acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo[i], xlo, acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi[i], xhi, acc[i][j], 0, 0, 0);
+            }
+        }
+
+        ++kk;
+        if (kk == KT) {
+            // ---- store the tile: lane holds n = n_base + 4*(l/16) + 0..3 at m = m_base + l%16
+            int tm, tn;
+            tile_coords(bid + cur_it * nblk, total_tiles, tiles_m, tiles_n, tm, tn);
+            const int m0 = tm * C::BM, n0 = tn * C::BN;
+            const int rows_left = M - m0;  // > 0
+            const int cols_left = N - n0;  // > 0
+            int32_t *ybase = Y + (size_t)m0 * N + n0;
+            // Byte extent of this tile's slab of C, measured from ybase.
+            const size_t slab_rows = rows_left < C::BM ? rows_left : C::BM;
+            const size_t extent = ((slab_rows - 1) * (size_t)N + (size_t)(cols_left < C::BN ? cols_left : C::BN)) * 4u;
+            __amdgpu_buffer_rsrc_t rsrc =
+                __builtin_amdgcn_make_buffer_rsrc(ybase, 0, (int)extent, 0x00020000);
+            // Offsets are split into a row part and a column part; a lane outside the
+            // matrix gets a part so large that the sum falls outside the descriptor's
+            // range and the hardware drops the store.
+            const int lm = opaque(wm * C::FM * 16 + fr);      // tile-relative m (plus j*16)
+            const int ln = opaque(wn * C::FN * 16 + fg * 4);  // tile-relative n (plus i*16)
+            unsigned col_off[C::FN];
+#pragma unroll
+            for (int i = 0; i < C::FN; ++i) {
+                const int ncol = ln + i * 16;
+                const bool ok = VEC_STORE ? (ncol + 3 < cols_left) : (ncol < cols_left);
+                col_off[i] = ok ? (unsigned)ncol * 4u : 0x40000000u;
+            }
+#pragma unroll
+            for (int j = 0; j < C::FM; ++j) {
+                const int mrow = lm + j * 16;
+                const unsigned row_off = mrow < rows_left ? (unsigned)mrow * (unsigned)N * 4u : 0x80000000u;
+#pragma unroll
+                for (int i = 0; i < C::FN; ++i) {
+                    const v4i v = acc[i][j] >> 8;
+                    if (VEC_STORE) {
+                        __builtin_amdgcn_raw_buffer_store_b128((v4u)v, rsrc, row_off + col_off[i], 0, 0);
+                    } else {
+                        // Element e of the four is valid while its column is inside the row.
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const int ncol = ln + i * 16 + e;
+                            const unsigned off = ncol < cols_left ? row_off + (unsigned)ncol * 4u : 0xC0000000u;
+                            __builtin_amdgcn_raw_buffer_store_b32((unsigned)v[e], rsrc, off, 0, 0);
+                        }
+                    }
+                }
+            }
+            kk = 0;
+            ++cur_it;
+        }
+    }
+}
+
+// 256 x 256 tile, four wavefronts of 128 x 128, one workgroup per CU: the large-shape
+// configuration (nibble widening is amortised over the largest wave tile the 512-entry
+// register file holds).
+using CfgLarge = TileConfig<2, 2, 8, 8, 4, 1>;
+// 128 x 128 tile, four wavefronts of 64 x 64, two workgroups per CU: mid-sized shapes
+// whose 256 x 256 tile count would leave CUs idle.
+using CfgMedium = TileConfig<2, 2, 4, 4, 4, 2>;
+
+template <class C>
+hipError_t set_lds_limit()
+{
+    hipError_t e = hipFuncSetAttribute((const void *)mfma_gemm_kernel<C, true>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+    if (e != hipSuccess)
+        return e;
+    return hipFuncSetAttribute((const void *)mfma_gemm_kernel<C, false>,
+                               hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+}
+
+template <class C>
+hipError_t launch_cfg(const void *a, const void *b, void *c, int m, int n, int k,
+                      const DeviceInfo &dev, hipStream_t stream)
+{
+    const int tiles_m = (m + C::BM - 1) / C::BM;
+    const int tiles_n = (n + C::BN - 1) / C::BN;
+    const long total = (long)tiles_m * tiles_n;
+    if (total > 0x7fffffffL)
+        return hipErrorInvalidValue;
+    long grid = (long)dev.cu_count * C::OCC;
+    if (grid > total)
+        grid = total;
+    // The epilogue addresses a tile's slab of C with 32-bit byte offsets.
+    if ((size_t)C::BM * (size_t)n * 4u > 0x40000000ull)
+        return hipErrorInvalidValue;
+    if (n % 4 == 0)
+        mfma_gemm_kernel<C, true><<<(unsigned)grid, C::THREADS, C::LDS_BYTES, stream>>>(
+            (const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k, tiles_m, tiles_n);
+    else
+        mfma_gemm_kernel<C, false><<<(unsigned)grid, C::THREADS, C::LDS_BYTES, stream>>>(
+            (const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k, tiles_m, tiles_n);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+bool mfma_supports(int m, int n, int k)
+{
+    // K <= 131071 keeps 256 * (sum of products) inside int32; one LDS row per stage is
+    // 128 nibbles; a row's byte offset inside a tile must fit 32 bits.
+    return m >= 1 && n >= 1 && k >= kStageK && k % kStageK == 0 && k <= 131071 - 127;
+}
+
+hipError_t mfma_init(const DeviceInfo &dev)
+{
+    if (dev.lds_per_cu < CfgLarge::LDS_BYTES)
+        return hipErrorInvalidConfiguration;
+    hipError_t e = set_lds_limit<CfgLarge>();
+    if (e != hipSuccess)
+        return e;
+    return set_lds_limit<CfgMedium>();
+}
+
+hipError_t launch_mfma(const void *a, const void *b, void *c, int m, int n, int k,
+                       const DeviceInfo &dev, hipStream_t stream)
+{
+    const long tiles_large = (long)((m + CfgLarge::BM - 1) / CfgLarge::BM) *
+                             ((n + CfgLarge::BN - 1) / CfgLarge::BN);
+    // Use the big tile once it alone can occupy every CU.
+    if (tiles_large >= dev.cu_count)
+        return launch_cfg<CfgLarge>(a, b, c, m, n, k, dev, stream);
+    return launch_cfg<CfgMedium>(a, b, c, m, n, k, dev, stream);
+}
+
+}  // namespace int4linear

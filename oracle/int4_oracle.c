@@ -1,0 +1,104 @@
+/*
+ * TEST INFRASTRUCTURE ONLY -- CPU oracle for the packed signed-int4 linear layer.
+ *
+ * This file restates, in plain C, the host-side algorithm of the reference
+ * (myeongs-song/Int4Linear).  It is the checker that the GPU library is compared
+ * against; it is never the thing that is shipped or measured as the product.
+ * Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may load it.
+ *
+ * Every function cites the reference lines it follows (paths relative to the
+ * reference tree).  How each one is pinned (none is "parity unpinned"):
+ *   oracle_pack        - known-answer words derived from utils/packer.cpp:11, a
+ *                        byte-view closed form, and a bit-for-bit diff against the
+ *                        reference's own packer.cpp compiled into oracle/_ref/.
+ *   oracle_unpack      - round trip through pack for every nibble value and ragged
+ *                        widths, nibble sign table, and the same diff against _ref.
+ *   oracle_linear_ref  - an independent float64 BLAS product (exact below 2^53),
+ *                        closed forms (all -8 => 64*K, one-hot rows, ones),
+ *                        algebraic invariants (linearity, K-permutation,
+ *                        transposition) and pure-Python brute force on tiny shapes.
+ *   oracle_is_same     - trivial; checked on equal / one-element-different arrays.
+ */
+#include <stddef.h>
+#include <stdint.h>
+
+/* utils/packer.cpp:3-18.  src holds one value per int (any int, only the low four
+ * bits are kept); dst holds ceil(n/8) 32-bit words per row; element 8j+k of a row
+ * goes to bits [4k, 4k+4) of word j; positions past n stay zero. */
+void oracle_pack(const int *src, int *dst, int m, int n)
+{
+    int words = (n + 7) / 8;
+    for (int row = 0; row < m; ++row) {
+        for (int w = 0; w < words; ++w) {
+            uint32_t word = 0;
+            for (int slot = 0; slot < 8; ++slot) {
+                int col = w * 8 + slot;
+                if (col < n) {
+                    uint32_t nib = (uint32_t)src[(size_t)row * n + col] & 0xFu;
+                    word |= nib << (4 * slot);
+                }
+            }
+            dst[(size_t)row * words + w] = (int)word;
+        }
+    }
+}
+
+/* utils/packer.cpp:20-31.  Inverse of pack; a nibble with bit 3 set is negative. */
+void oracle_unpack(const int *src, int *dst, int m, int n)
+{
+    int words = (n + 7) / 8;
+    for (int row = 0; row < m; ++row) {
+        for (int col = 0; col < n; ++col) {
+            uint32_t word = (uint32_t)src[(size_t)row * words + col / 8];
+            int nib = (int)((word >> (4 * (col % 8))) & 0xFu);
+            dst[(size_t)row * n + col] = (nib >= 8) ? nib - 16 : nib;
+        }
+    }
+}
+
+/* test/test_correctness.cu:12-19.  y[i][j] = sum_l x[i][l] * w[j][l] over UNPACKED
+ * int-per-element arrays, int32 accumulation, i-j-l loop order. */
+void oracle_linear_ref(const int *x, const int *w, int *y, int m, int n, int k)
+{
+    for (int i = 0; i < m; ++i) {
+        const int *xr = x + (size_t)i * k;
+        for (int j = 0; j < n; ++j) {
+            const int *wr = w + (size_t)j * k;
+            int acc = 0;
+            for (int l = 0; l < k; ++l)
+                acc += xr[l] * wr[l];
+            y[(size_t)i * n + j] = acc;
+        }
+    }
+}
+
+/* Same loop nest as oracle_linear_ref with the outer (row) loop spread over
+ * `threads` OpenMP threads.  Used for the "all host cores" CPU baseline and to keep
+ * full-matrix checks of mid-sized shapes within seconds.  Integer sums make the
+ * result independent of the thread count. */
+void oracle_linear_ref_mt(const int *x, const int *w, int *y, int m, int n, int k,
+                          int threads)
+{
+    if (threads < 1)
+        threads = 1;
+#pragma omp parallel for num_threads(threads) schedule(dynamic, 1)
+    for (int i = 0; i < m; ++i) {
+        const int *xr = x + (size_t)i * k;
+        for (int j = 0; j < n; ++j) {
+            const int *wr = w + (size_t)j * k;
+            int acc = 0;
+            for (int l = 0; l < k; ++l)
+                acc += xr[l] * wr[l];
+            y[(size_t)i * n + j] = acc;
+        }
+    }
+}
+
+/* test/test_correctness.cu:22-27.  1 when the first `count` ints agree, else 0. */
+int oracle_is_same(const int *a, const int *b, int count)
+{
+    for (int i = 0; i < count; ++i)
+        if (a[i] != b[i])
+            return 0;
+    return 1;
+}

@@ -1,0 +1,30 @@
+import os
+import sys
+from pathlib import Path
+
+import pytest
+
+ROOT = Path(__file__).resolve().parent.parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (gfx950) device")
+
+
+@pytest.fixture(scope="session")
+def gpu():
+    """Device handle for GPU tests; fails (not skips) if the HIP library is missing."""
+    import torch
+
+    assert torch.cuda.is_available(), "GPU test selected but no HIP device is visible"
+    import int4linear_amd
+
+    int4linear_amd.init()
+    return torch.device("cuda:0")
+
+
+@pytest.fixture(scope="session")
+def host_threads():
+    return max(1, min(16, os.cpu_count() or 1))

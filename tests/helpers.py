@@ -1,0 +1,71 @@
+"""Shared test helpers: seeded inputs, packing, and the C-ABI call wrapper."""
+from __future__ import annotations
+
+import numpy as np
+
+from oracle import loader as oracle
+
+
+def uniform_s4(seed: int, rows: int, cols: int) -> np.ndarray:
+    """Uniform integers in [-8, 7], int8, from a fixed seed."""
+    rng = np.random.default_rng(seed)
+    return rng.integers(-8, 8, size=(rows, cols), dtype=np.int8)
+
+
+def normal_s4(seed: int, rows: int, cols: int, sigma: float = 2.0) -> np.ndarray:
+    """normal(0, sigma) rounded to nearest and clamped to [-8, 7] (decode activations)."""
+    rng = np.random.default_rng(seed)
+    v = np.rint(rng.normal(0.0, sigma, size=(rows, cols)))
+    return np.clip(v, -8, 7).astype(np.int8)
+
+
+def pack_bytes(values: np.ndarray) -> np.ndarray:
+    """(m, k) int8/int32 in [-8,7] with k % 2 == 0 -> (m, k/2) uint8, low nibble = even k.
+    Vectorised numpy restatement of the byte view of the packer; checked against the
+    oracle's pack in the CPU tests."""
+    v = values.astype(np.uint8) & 0xF
+    return (v[:, 0::2] | (v[:, 1::2] << 4)).astype(np.uint8)
+
+
+def pack_words_as_bytes(values: np.ndarray) -> np.ndarray:
+    """Same bytes via the oracle's word packer (little-endian host)."""
+    return oracle.pack(values.astype(np.int32)).view(np.uint8)
+
+
+def exact_matmul(x: np.ndarray, w: np.ndarray) -> np.ndarray:
+    """Independent implementation: float64 BLAS product, exact while |sum| < 2^53."""
+    y = x.astype(np.float64) @ w.astype(np.float64).T
+    assert np.all(np.abs(y) < 2.0 ** 31)
+    return y.astype(np.int64).astype(np.int32)
+
+
+GUARD_WORDS = 16384  # int32 words of poison kept before and after C
+
+
+def run_gemm(xp: np.ndarray, wp: np.ndarray, m: int, n: int, k: int, kernel: str = "auto",
+             poison: int = 0x5A5A5A5A, keep_on_device: bool = False):
+    """Copy packed operands to the device, run the C-ABI GEMM, return C as numpy int32
+    (or the device tensor).  C sits between two guard zones and everything is pre-filled
+    with a poison value, so untouched outputs and out-of-bounds writes are both caught."""
+    import torch
+
+    import int4linear_amd as lib
+
+    dev = torch.device("cuda:0")
+    xd = torch.from_numpy(np.ascontiguousarray(xp).view(np.uint8).reshape(-1)).to(dev)
+    wd = torch.from_numpy(np.ascontiguousarray(wp).view(np.uint8).reshape(-1)).to(dev)
+    buf = torch.full((2 * GUARD_WORDS + m * n,), poison, dtype=torch.int32, device=dev)
+    yd = buf[GUARD_WORDS:GUARD_WORDS + m * n].view(m, n)
+    lib.gemm_s4s4s32(xd, wd, yd, m, n, k, kernel=kernel)
+    torch.cuda.synchronize()
+    assert bool((buf[:GUARD_WORDS] == poison).all()), "write before the start of C"
+    assert bool((buf[GUARD_WORDS + m * n:] == poison).all()), "write past the end of C"
+    if keep_on_device:
+        return yd
+    return yd.cpu().numpy()
+
+
+def to_device_bytes(packed: np.ndarray):
+    import torch
+
+    return torch.from_numpy(np.ascontiguousarray(packed).view(np.uint8).reshape(-1)).to("cuda:0")

@@ -1,0 +1,232 @@
+"""GPU parity tests: every kernel of the library, called through the C ABI, against the
+CPU oracle on identical seeded inputs -- bit-exact int32.  Covers the five benchmark
+configurations, the committed golden vectors, ragged and degenerate shapes, and
+size-independent properties at full size."""
+import numpy as np
+import pytest
+
+from oracle import loader as oracle
+from tests import helpers
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = np.load(helpers.__file__.replace("helpers.py", "golden/int4_gemm_golden.npz"))
+
+
+def kernels_for(m, n, k):
+    ks = ["auto", "simple"]
+    if k >= 128 and k % 128 == 0:
+        ks.append("mfma")
+        if m <= 64:
+            ks.append("skinny")
+    return ks
+
+
+def check_all_kernels(x, w, want=None, threads=1, kernels=None):
+    m, k = x.shape
+    n = w.shape[0]
+    if want is None:
+        want = oracle.linear_ref(x, w, threads=threads)
+    xp, wp = helpers.pack_words_as_bytes(x), helpers.pack_words_as_bytes(w)
+    for kern in kernels or kernels_for(m, n, k):
+        got = helpers.run_gemm(xp, wp, m, n, k, kernel=kern)
+        bad = np.argwhere(got != want)
+        assert bad.size == 0, (f"kernel={kern} shape={(m, n, k)}: {len(bad)} mismatches, first at "
+                               f"{tuple(bad[0])}: got {got[tuple(bad[0])]} want {want[tuple(bad[0])]}")
+
+
+# ---- committed golden vectors ----------------------------------------------------------
+
+@pytest.mark.parametrize("idx", range(len(GOLDEN["shapes"])))
+def test_golden_vectors(gpu, idx):
+    x, w, y = GOLDEN[f"x{idx}"], GOLDEN[f"w{idx}"], GOLDEN[f"y{idx}"]
+    check_all_kernels(x, w, want=y)
+
+
+# ---- configuration 1: 1024^3, full compare ---------------------------------------------
+
+def test_cfg1_1024_cubed(gpu, host_threads):
+    x = helpers.uniform_s4(1, 1024, 1024)
+    w = helpers.uniform_s4(2, 1024, 1024)
+    check_all_kernels(x, w, threads=host_threads)
+
+
+# ---- configurations 2 and 3: large squares and the 2M = 2N = K family ------------------
+
+@pytest.mark.parametrize("m, n, k", [
+    (2048, 2048, 2048), (4096, 4096, 4096), (8192, 8192, 8192),
+    (1024, 1024, 2048), (2048, 2048, 4096), (4096, 4096, 8192),
+])
+def test_cfg2_cfg3_large(gpu, host_threads, m, n, k):
+    import torch
+
+    x = helpers.uniform_s4(100 + m, m, k)
+    w = helpers.uniform_s4(200 + k, n, k)
+    xp, wp = helpers.pack_bytes(x), helpers.pack_bytes(w)
+    got_d = helpers.run_gemm(xp, wp, m, n, k, kernel="auto", keep_on_device=True)
+    # sampled rows against the CPU oracle
+    rows = np.unique(np.concatenate([[0, 1, m - 1, 255, 256], np.random.default_rng(m + k).integers(0, m, 27)]))
+    want = oracle.linear_ref(x[rows], w, threads=host_threads)
+    got_rows = got_d[torch.from_numpy(rows).to(got_d.device)].cpu().numpy()
+    assert np.array_equal(got_rows, want)
+    # the whole matrix against the independent scalar kernel, on the device
+    ref_d = helpers.run_gemm(xp, wp, m, n, k, kernel="simple", keep_on_device=True)
+    assert torch.equal(got_d, ref_d)
+
+
+# ---- configuration 4: decode shapes ------------------------------------------------------
+
+@pytest.mark.parametrize("n, k", [(4096, 4096), (14336, 4096), (4096, 14336)])
+@pytest.mark.parametrize("m", [1, 16, 64])
+def test_cfg4_decode(gpu, host_threads, m, n, k):
+    x = helpers.normal_s4(300 + m, m, k)           # activations: normal(0, 2) -> [-8, 7]
+    w = helpers.uniform_s4(400 + n + k, n, k)      # weights: uniform [-8, 7]
+    want = oracle.linear_ref(x, w, threads=host_threads)
+    xp, wp = helpers.pack_bytes(x), helpers.pack_bytes(w)
+    for kern in ("auto", "skinny", "mfma"):
+        got = helpers.run_gemm(xp, wp, m, n, k, kernel=kern)
+        assert np.array_equal(got, want), f"kernel={kern}"
+
+
+# ---- configuration 5: adversarial ---------------------------------------------------------
+
+def test_cfg5_all_minus_eight_full_size(gpu):
+    import torch
+
+    m, n, k = 8192, 28672, 8192
+    xp = np.full((m, k // 2), 0x88, dtype=np.uint8)
+    wp = np.full((n, k // 2), 0x88, dtype=np.uint8)
+    got = helpers.run_gemm(xp, wp, m, n, k, kernel="auto", keep_on_device=True)
+    assert bool((got == 524288).all())
+    assert int(got.min()) == 524288 and int(got.max()) == 524288
+    del got
+    torch.cuda.empty_cache()
+
+
+def test_cfg5_ragged_1000_3000_4096(gpu, host_threads):
+    x = helpers.uniform_s4(51, 1000, 4096)
+    w = helpers.uniform_s4(52, 3000, 4096)
+    check_all_kernels(x, w, threads=host_threads, kernels=["auto", "mfma", "simple"])
+
+
+@pytest.mark.parametrize("a, b, per_k", [(-8, -8, 64), (7, 7, 49), (-8, 7, -56), (7, -8, -56)])
+def test_extreme_constants(gpu, a, b, per_k):
+    m, n, k = 300, 260, 8192
+    x = np.full((m, k), a, dtype=np.int8)
+    w = np.full((n, k), b, dtype=np.int8)
+    check_all_kernels(x, w, want=np.full((m, n), per_k * k, dtype=np.int32))
+
+
+# ---- edges ------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("m, n, k", [
+    (1, 1, 128), (15, 17, 128), (16, 16, 256), (65, 3, 384), (257, 255, 128), (256, 256, 512),
+    (129, 130, 640), (300, 515, 256), (513, 257, 1024), (70, 1000, 1152), (2, 2, 8), (9, 7, 24),
+    (31, 33, 72), (64, 64, 64), (100, 100, 200),
+])
+def test_ragged_shapes(gpu, m, n, k):
+    x = helpers.uniform_s4(m * 7 + n, m, k)
+    w = helpers.uniform_s4(k * 3 + n, n, k)
+    check_all_kernels(x, w, threads=4)
+
+
+def test_one_hot_rows_pin_nibble_and_k_order(gpu):
+    # W[j] = delta(l, k_j)  =>  C[i][j] = A[i][k_j], for every k position of several stages.
+    m, k = 40, 512
+    n = k
+    x = helpers.uniform_s4(61, m, k)
+    w = np.zeros((n, k), dtype=np.int8)
+    w[np.arange(n), np.arange(n)] = 1
+    check_all_kernels(x, w, want=x.astype(np.int32))
+
+
+def test_degenerate_sizes(gpu):
+    import torch
+
+    import int4linear_amd as lib
+
+    dev = torch.device("cuda:0")
+    y = torch.full((8, 12), 77, dtype=torch.int32, device=dev)
+    a = torch.zeros(64, dtype=torch.uint8, device=dev)
+    lib.gemm_s4s4s32(a, a, y, 8, 12, 0)             # K == 0: C is zero-filled
+    torch.cuda.synchronize()
+    assert not bool(y.any())
+    y.fill_(77)
+    lib.gemm_s4s4s32(a, a, y, 0, 12, 128)           # M == 0: nothing happens
+    lib.gemm_s4s4s32(a, a, y, 8, 0, 128)            # N == 0: nothing happens
+    torch.cuda.synchronize()
+    assert bool((y == 77).all())
+    with pytest.raises(lib.Int4LinearError):
+        lib.gemm_s4s4s32(a, a, y, 8, 12, 64, kernel="mfma")   # K below one stage
+    with pytest.raises(lib.Int4LinearError):
+        lib.gemm_s4s4s32(a, a, y, 65, 12, 128, kernel="skinny")  # M too large
+
+
+# ---- properties that hold at any size -------------------------------------------------------
+
+def test_properties_at_4096(gpu):
+    import torch
+
+    m = n = k = 4096
+    x = helpers.uniform_s4(71, m, k)
+    w = helpers.uniform_s4(72, n, k)
+    xp, wp = helpers.pack_bytes(x), helpers.pack_bytes(w)
+    y = helpers.run_gemm(xp, wp, m, n, k, keep_on_device=True)
+    # swapping the operands transposes the result
+    yt = helpers.run_gemm(wp, xp, n, m, k, keep_on_device=True)
+    assert torch.equal(yt, y.t())
+    # the same byte permutation along K on both operands changes nothing
+    perm = np.random.default_rng(73).permutation(k // 2)
+    yp = helpers.run_gemm(xp[:, perm], wp[:, perm], m, n, k, keep_on_device=True)
+    assert torch.equal(yp, y)
+    # negating A (values in [-7, 7] so -A is representable) negates C
+    x7 = np.clip(x, -7, 7)
+    y7 = helpers.run_gemm(helpers.pack_bytes(x7), wp, m, n, k, keep_on_device=True)
+    yn = helpers.run_gemm(helpers.pack_bytes(-x7), wp, m, n, k, keep_on_device=True)
+    assert torch.equal(yn, -y7)
+    # row sums: A = ones  =>  C[i][j] = sum_l W[j][l]
+    ones = helpers.pack_bytes(np.ones((64, k), dtype=np.int8))
+    ys = helpers.run_gemm(ones, wp, 64, n, k)
+    assert np.array_equal(ys, np.tile(w.astype(np.int32).sum(axis=1), (64, 1)))
+
+
+# ---- the reference's blocking entry points ------------------------------------------------------
+
+@pytest.mark.parametrize("version", [0, 1, 2, 10, 11, 20, 21])
+def test_reference_entry_points(gpu, version):
+    import torch
+
+    import int4linear_amd as lib
+
+    m, n, k = 260, 136, 256
+    x = helpers.uniform_s4(80 + version, m, k)
+    w = helpers.uniform_s4(90 + version, n, k)
+    want = oracle.linear_ref(x, w)
+    # operands packed by the library's own host packer, as the reference's harness does
+    xd = helpers.to_device_bytes(lib.pack_rows(x))
+    wd = helpers.to_device_bytes(lib.pack_rows(w))
+    yd = torch.full((m, n), -1, dtype=torch.int32, device="cuda:0")
+    getattr(lib, f"linear_v{version}_launch")(xd, wd, yd, m, n, k)
+    # blocking call: the result is complete on return, no synchronisation here
+    assert oracle.is_same(yd.cpu().numpy(), want)
+
+
+# ---- device packer / unpacker ----------------------------------------------------------------------
+
+@pytest.mark.parametrize("m, n", [(1, 8), (5, 13), (64, 4096), (33, 1001), (1000, 64)])
+def test_device_packer(gpu, m, n):
+    import torch
+
+    import int4linear_amd as lib
+
+    v = np.random.default_rng(m + n).integers(-100, 100, size=(m, n), dtype=np.int32)
+    words = (n + 7) // 8
+    src = torch.from_numpy(v).to("cuda:0")
+    dst = torch.full((m, words), -1, dtype=torch.int32, device="cuda:0")
+    lib.pack_device(src, dst, m, n)
+    back = torch.full((m, n), 99, dtype=torch.int32, device="cuda:0")
+    lib.unpack_device(dst, back, m, n)
+    torch.cuda.synchronize()
+    want_words = oracle.pack(v)
+    assert np.array_equal(dst.cpu().numpy(), want_words)
+    assert np.array_equal(back.cpu().numpy(), oracle.unpack(want_words, n))

@@ -1,0 +1,103 @@
+"""Pins oracle_linear_ref (restating test/test_correctness.cu:12-19) and oracle_is_same
+(:22-27) with checks that do not retype its formula: committed golden products, an
+independent float64 BLAS product, closed forms, algebraic invariants and a pure-Python
+brute force.  A dropped term, a wrong sign or index, or a transposed operand fails at
+least one of them."""
+import numpy as np
+import pytest
+
+from oracle import loader as oracle
+from tests import helpers
+
+GOLDEN = np.load(helpers.__file__.replace("helpers.py", "golden/int4_gemm_golden.npz"))
+
+
+def test_golden_products():
+    for idx, (m, n, k) in enumerate(GOLDEN["shapes"]):
+        y = oracle.linear_ref(GOLDEN[f"x{idx}"], GOLDEN[f"w{idx}"])
+        assert y.shape == (m, n)
+        assert np.array_equal(y, GOLDEN[f"y{idx}"]), f"case {idx} {(m, n, k)}"
+
+
+@pytest.mark.parametrize("m, n, k, seed", [(64, 96, 256, 1), (37, 53, 1000, 2), (128, 128, 1024, 3)])
+def test_against_blas_float64(m, n, k, seed):
+    x = helpers.uniform_s4(seed, m, k)
+    w = helpers.uniform_s4(seed + 100, n, k)
+    assert np.array_equal(oracle.linear_ref(x, w), helpers.exact_matmul(x, w))
+
+
+def test_threaded_variant_matches_single_thread():
+    x = helpers.uniform_s4(5, 50, 512)
+    w = helpers.uniform_s4(6, 70, 512)
+    assert np.array_equal(oracle.linear_ref(x, w, threads=4), oracle.linear_ref(x, w))
+
+
+@pytest.mark.parametrize("a, b, per_k", [(-8, -8, 64), (7, 7, 49), (-8, 7, -56), (1, -1, -1)])
+def test_constant_operands(a, b, per_k):
+    m, n, k = 5, 6, 4096
+    y = oracle.linear_ref(np.full((m, k), a), np.full((n, k), b))
+    assert np.all(y == per_k * k)
+
+
+def test_all_minus_eight_at_k_8192_is_524288():
+    y = oracle.linear_ref(np.full((2, 8192), -8), np.full((3, 8192), -8))
+    assert np.all(y == 524288)
+
+
+def test_one_hot_rows_select_columns():
+    # W[j] = delta(l, k_j)  =>  C[i][j] = A[i][k_j]; pins the k index and the B-row index.
+    m, n, k = 9, 11, 64
+    x = helpers.uniform_s4(8, m, k).astype(np.int32)
+    kj = (np.arange(n) * 7 + 3) % k
+    w = np.zeros((n, k), dtype=np.int32)
+    w[np.arange(n), kj] = 1
+    assert np.array_equal(oracle.linear_ref(x, w), x[:, kj])
+
+
+def test_ones_give_row_sums():
+    n, k = 13, 200
+    w = helpers.uniform_s4(9, n, k).astype(np.int32)
+    y = oracle.linear_ref(np.ones((4, k), dtype=np.int32), w)
+    assert np.array_equal(y, np.tile(w.sum(axis=1), (4, 1)))
+
+
+def test_invariants():
+    m, n, k = 12, 10, 96
+    x = helpers.uniform_s4(10, m, k).astype(np.int32)
+    x2 = helpers.uniform_s4(11, m, k).astype(np.int32)
+    w = helpers.uniform_s4(12, n, k).astype(np.int32)
+    y = oracle.linear_ref(x, w)
+    # linear in A
+    assert np.array_equal(oracle.linear_ref(x + x2, w), y + oracle.linear_ref(x2, w))
+    # the same K permutation on both operands changes nothing
+    perm = np.random.default_rng(13).permutation(k)
+    assert np.array_equal(oracle.linear_ref(x[:, perm], w[:, perm]), y)
+    # swapping operands transposes the result
+    assert np.array_equal(oracle.linear_ref(w, x), y.T)
+    # permuting rows of A / rows of B permutes rows / columns of C
+    pr, pc = np.random.default_rng(14).permutation(m), np.random.default_rng(15).permutation(n)
+    assert np.array_equal(oracle.linear_ref(x[pr], w[pc]), y[pr][:, pc])
+
+
+@pytest.mark.parametrize("m, n, k", [(1, 1, 8), (2, 3, 8), (3, 2, 24), (4, 4, 32)])
+def test_brute_force_python(m, n, k):
+    x = helpers.uniform_s4(20 + m, m, k)
+    w = helpers.uniform_s4(30 + n, n, k)
+    want = [[sum(int(x[i, l]) * int(w[j, l]) for l in range(k)) for j in range(n)] for i in range(m)]
+    assert oracle.linear_ref(x, w).tolist() == want
+
+
+def test_empty_k_gives_zeros():
+    y = oracle.linear_ref(np.zeros((3, 0), dtype=np.int32), np.zeros((4, 0), dtype=np.int32))
+    assert y.shape == (3, 4) and not y.any()
+
+
+def test_is_same():
+    a = np.arange(100, dtype=np.int32)
+    b = a.copy()
+    assert oracle.is_same(a, b)
+    b[99] += 1
+    assert not oracle.is_same(a, b)
+    b[99] -= 1
+    b[0] -= 1
+    assert not oracle.is_same(a, b)
