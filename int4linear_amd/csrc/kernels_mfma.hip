@@ -1,7 +1,7 @@
 // LDS-pipelined int8-MFMA GEMM over packed signed-int4 operands for gfx950 (CDNA4).
 //
 // gfx950 has no 4-bit integer MFMA, so nibbles are widened to int8 in registers and fed
-// to v_mfma_i32_16x16x64_i8.  The widening keeps each nibble in the HIGH half of its
+// to v_mfma_i32_32x32x32_i8.  The widening keeps each nibble in the HIGH half of its
 // byte: for a packed word w,  (w << 4) & 0xF0F0F0F0  holds the even-k nibbles and
 // w & 0xF0F0F0F0 the odd-k nibbles, each as the signed byte 16*value (the nibble's own
 // sign bit lands in bit 7, so no sign-extension step exists).  Both operands carry the
@@ -16,11 +16,12 @@
 //   HBM/L2 --global_load_lds_dwordx4 (16 B per lane, straight into LDS)--> NSTAGE-deep ring
 //   LDS    --ds_read_b128 (bank-conflict-free through a 16-byte-chunk XOR swizzle)--> VGPRs
 //   VGPRs  --3 VALU ops per packed dword--> int8 operands --MFMA--> int32 accumulators
-//   accumulators --buffer_store_dwordx4 (W is the MFMA A operand, so a lane's four
-//                 accumulators are four consecutive n)--> C
-// The kernel is persistent: gridDim.x workgroups walk a list of tiles, and the load
-// ring runs NSTAGE-1 stages ahead of the math ACROSS tile boundaries, so the next
-// tile's first stages are in flight while the current tile stores C.
+//   accumulators --buffer_store_dwordx4 (W is the MFMA A operand, so each quad of a
+//                 lane's accumulators is four consecutive n)--> C
+// Two wavefronts share each SIMD: while one widens nibbles on the VALU the other keeps
+// the matrix pipe busy.  The kernel is persistent: gridDim.x workgroups walk a list of
+// tiles, and the load ring runs NSTAGE-1 stages ahead of the math ACROSS tile
+// boundaries, so the next tile's first stages are in flight while this tile stores C.
 #include "kernels.h"
 
 namespace int4linear {
@@ -28,6 +29,7 @@ namespace int4linear {
 namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
 typedef unsigned v4u __attribute__((ext_vector_type(4)));
 
 #define I4L_LDS(p) ((__attribute__((address_space(3))) void *)(p))
@@ -61,35 +63,37 @@ constexpr int kStageK = 128;                 // nibbles of K per pipeline stage
 constexpr int kRowBytes = kStageK / 2;       // bytes per LDS row (64)
 constexpr int kChunkRows = 16;               // rows moved by one 64-lane 16-byte load
 constexpr int kChunkBytes = kChunkRows * kRowBytes;  // 1 KiB
+constexpr int kFrag = 32;                    // rows of an MFMA 32x32x32 operand
 
 // Tile configuration.  A workgroup is WAVES_M x WAVES_N wavefronts; each owns
-// FM x FN MFMA tiles of 16x16, i.e. a (FM*16) x (FN*16) patch of C.
+// FM x FN MFMA tiles of 32x32, i.e. a (FM*32) x (FN*32) patch of C.
 template <int WAVES_M_, int WAVES_N_, int FM_, int FN_, int NSTAGE_, int OCC_>
 struct TileConfig {
     static constexpr int WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
     static constexpr int FM = FM_, FN = FN_;
     static constexpr int NSTAGE = NSTAGE_;
-    static constexpr int OCC = OCC_;  // workgroups per CU the register budget allows
+    static constexpr int OCC = OCC_;  // workgroups per CU
     static constexpr int NWAVES = WAVES_M * WAVES_N;
     static constexpr int THREADS = NWAVES * 64;
-    static constexpr int BM = WAVES_M * FM * 16;
-    static constexpr int BN = WAVES_N * FN * 16;
+    static constexpr int BM = WAVES_M * FM * kFrag;
+    static constexpr int BN = WAVES_N * FN * kFrag;
     static constexpr int X_CHUNKS = BM / kChunkRows;
     static constexpr int W_CHUNKS = BN / kChunkRows;
     static constexpr int CH = (X_CHUNKS + W_CHUNKS) / NWAVES;  // loads per wave per stage
     static constexpr int X_CH = X_CHUNKS / NWAVES;             // of which from X
     static constexpr int STAGE_BYTES = (BM + BN) * kRowBytes;
     static constexpr int LDS_BYTES = STAGE_BYTES * NSTAGE;
-    static constexpr int STORES = FM * FN;  // dwordx4 stores per lane per tile
+    static constexpr int STORES = FM * FN * 4;  // dwordx4 stores per lane per tile
     static_assert(X_CHUNKS % NWAVES == 0 && W_CHUNKS % NWAVES == 0, "chunks must split evenly");
-    static_assert((NSTAGE - 2) * CH <= 63, "vmcnt is six bits");
+    static_assert((NSTAGE - 2) * CH + STORES <= 63, "vmcnt is six bits");
 };
 
-// Which 16-byte slot of its 64-byte LDS row holds logical chunk g of row r:  g ^ swz(r).
-// With rows 64 B apart, sixteen lanes reading the same g of rows 0..15 touch sixteen
-// different 16-byte bank groups of a 256-byte window, and any eight consecutive of them
-// touch eight different groups of a 128-byte window.
-__device__ __forceinline__ int swz(int r) { return ((r >> 1) + (r >> 3)) & 3; }
+// Which 16-byte slot of its 64-byte LDS row holds logical chunk c of row r:  c ^ swz(r),
+// a function of r mod 16 (the rows one 64-lane load moves).
+// With rows 64 B apart, sixteen lanes reading the same c of sixteen consecutive rows
+// touch sixteen different 16-byte bank groups of a 256-byte window, and any aligned
+// eight of them touch eight different groups of a 128-byte window.
+__device__ __forceinline__ int swz(int r) { r &= 15; return ((r >> 1) + (r >> 3)) & 3; }
 
 // Tile order.  Workgroup ids go round-robin over the 8 XCDs, each with a private L2, so
 // the tiles that run together on one XCD (ids congruent mod 8, consecutive quotients)
@@ -136,11 +140,10 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
     // ---- load side -------------------------------------------------------------------
     // Lane p of a chunk lands at LDS byte p*16 of that chunk: row p/4, slot p%4.
     const int ld_row = lane >> 2;
-    const int ld_g = (lane & 3) ^ swz(ld_row);
-    unsigned voff[C::CH];            // per-chunk byte offset of this lane from the tile base
+    const int ld_c = (lane & 3) ^ swz(ld_row);
+    unsigned voff[C::CH];                // per-chunk byte offset of this lane from the tile base
     const uint8_t *xptr = X, *wptr = W;  // wave-uniform: tile base + k offset
     int ld_it = 0, ld_k = 0, issued = 0;
-
     const unsigned lds_base = (unsigned)(size_t)I4L_LDS(lds);
 
     auto ld_setup_tile = [&](int it) {
@@ -155,7 +158,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
             const int r = ci * kChunkRows + row;
             const int lim = is_x ? (M - 1 - m0) : (N - 1 - n0);  // last valid row, tile-relative
             const int rc = r < lim ? r : lim;
-            voff[c] = (unsigned)rc * (unsigned)rowbytes + (unsigned)ld_g * 16u;
+            voff[c] = (unsigned)rc * (unsigned)rowbytes + (unsigned)ld_c * 16u;
         }
         xptr = X + (size_t)m0 * rowbytes;
         wptr = W + (size_t)n0 * rowbytes;
@@ -190,15 +193,22 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
             ld_issue();
 
     // ---- math side -------------------------------------------------------------------
-    // Lane l of a 16x16x64 MFMA supplies row l%16, k-chunk l/16 of both operands.
-    const int fr = lane & 15;
-    const int fg = lane >> 4;
-    const unsigned rd_off = (unsigned)fr * kRowBytes + (unsigned)((fg ^ swz(fr)) * 16);
-    const unsigned x_rd = rd_off + (unsigned)(wm * C::FM * 16 * kRowBytes);
-    const unsigned w_rd = rd_off + (unsigned)(C::BM * kRowBytes + wn * C::FN * 16 * kRowBytes);
+    // Lane l of a 32x32x32 MFMA supplies row l%32 and 16 of the 32 k values of both
+    // operands.  A 16-byte LDS read holds 32 nibbles: the even ones feed one MFMA, the odd
+    // ones the next.  Half h of a stage is the two 16-byte chunks 2h and 2h+1 of a row,
+    // one per 32-lane group.
+    const int fr = lane & 31;
+    const int fg = lane >> 5;
+    const int fsw = swz(fr);
+    unsigned rd_off[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+        rd_off[h] = (unsigned)fr * kRowBytes + (unsigned)(((2 * h + fg) ^ fsw) * 16);
+    const unsigned x_rd = (unsigned)(wm * C::FM * kFrag * kRowBytes);
+    const unsigned w_rd = (unsigned)(C::BM * kRowBytes + wn * C::FN * kFrag * kRowBytes);
     const int himask = (int)0xF0F0F0F0u;
 
-    v4i acc[C::FN][C::FM];
+    v16i acc[C::FN][C::FM];
     int cur_it = 0, kk = 0;
 
 #pragma unroll 1
@@ -209,7 +219,8 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
         const int ahead = issued - 1 - gs;
         if (ahead >= C::NSTAGE - 2) {
             if (cur_it > 0 && kk < C::NSTAGE - 1) {
-                constexpr int with_stores = (C::NSTAGE - 2) * C::CH + (VEC_STORE ? C::STORES : 64);
+                constexpr int stores = VEC_STORE ? C::STORES : 4 * C::STORES;
+                constexpr int with_stores = (C::NSTAGE - 2) * C::CH + stores;
                 __builtin_amdgcn_s_waitcnt(I4L_VMCNT(with_stores < 63 ? with_stores : 63));
             } else {
                 __builtin_amdgcn_s_waitcnt(I4L_VMCNT((C::NSTAGE - 2) * C::CH));
@@ -229,35 +240,41 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
             for (int i = 0; i < C::FN; ++i)
 #pragma unroll
                 for (int j = 0; j < C::FM; ++j)
-                    acc[i][j] = (v4i){0, 0, 0, 0};
+#pragma unroll
+                    for (int t = 0; t < 16; ++t)
+                        acc[i][j][t] = 0;
         }
 
         const uint8_t *stage = lds + (gs % C::NSTAGE) * C::STAGE_BYTES;
-        // W fragments are widened once per stage and stay live; X fragments stream
-        // through one at a time, which bounds the operand registers next to the
-        // FM*FN*4 accumulators.
-        v4i wlo[C::FN], whi[C::FN];
 #pragma unroll
-        for (int i = 0; i < C::FN; ++i) {
-            const v4i ww = *(const v4i *)(stage + w_rd + i * 16 * kRowBytes);
-            wlo[i] = (ww << 4) & himask;  // even-k nibbles
-            whi[i] = ww & himask;         // odd-k nibbles
-        }
-#pragma unroll
-        for (int j = 0; j < C::FM; ++j) {
-            const v4i xw = *(const v4i *)(stage + x_rd + j * 16 * kRowBytes);
-            const v4i xlo = (xw << 4) & himask;
-            const v4i xhi = xw & himask;
+        for (int h = 0; h < 2; ++h) {
+            // W fragments of this half are widened once and stay live; X fragments
+            // stream through.
+            v4i wlo[C::FN], whi[C::FN];
 #pragma unroll
             for (int i = 0; i < C::FN; ++i) {
-                acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo[i], xlo, acc[i][j], 0, 0, 0);
-                acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi[i], xhi, acc[i][j], 0, 0, 0);
+                const v4i ww = *(const v4i *)(stage + w_rd + rd_off[h] + i * kFrag * kRowBytes);
+                wlo[i] = (ww << 4) & himask;  // even-k nibbles
+                whi[i] = ww & himask;         // odd-k nibbles
+            }
+#pragma unroll
+            for (int j = 0; j < C::FM; ++j) {
+                const v4i xw = *(const v4i *)(stage + x_rd + rd_off[h] + j * kFrag * kRowBytes);
+                const v4i xlo = (xw << 4) & himask;
+                const v4i xhi = xw & himask;
+#pragma unroll
+                for (int i = 0; i < C::FN; ++i)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wlo[i], xlo, acc[i][j], 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < C::FN; ++i)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(whi[i], xhi, acc[i][j], 0, 0, 0);
             }
         }
 
         ++kk;
         if (kk == KT) {
-            // ---- store the tile: lane holds n = n_base + 4*(l/16) + 0..3 at m = m_base + l%16
+            // ---- store the tile.  Accumulator t of MFMA tile (i, j) belongs to
+            //      n = 32*i + 8*(t/4) + 4*(lane/32) + t%4,  m = 32*j + lane%32.
             int tm, tn;
             tile_coords(bid + cur_it * nblk, total_tiles, tiles_m, tiles_n, tm, tn);
             const int m0 = tm * C::BM, n0 = tn * C::BN;
@@ -272,31 +289,30 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
             // Offsets are split into a row part and a column part; a lane outside the
             // matrix gets a part so large that the sum falls outside the descriptor's
             // range and the hardware drops the store.
-            const int lm = opaque(wm * C::FM * 16 + fr);      // tile-relative m (plus j*16)
-            const int ln = opaque(wn * C::FN * 16 + fg * 4);  // tile-relative n (plus i*16)
-            unsigned col_off[C::FN];
-#pragma unroll
-            for (int i = 0; i < C::FN; ++i) {
-                const int ncol = ln + i * 16;
-                const bool ok = VEC_STORE ? (ncol + 3 < cols_left) : (ncol < cols_left);
-                col_off[i] = ok ? (unsigned)ncol * 4u : 0x40000000u;
-            }
+            const int lm = opaque(wm * C::FM * kFrag + fr);      // tile-relative m (plus 32*j)
+            const int ln = opaque(wn * C::FN * kFrag + fg * 4);  // tile-relative n (plus 32*i + 8*q)
 #pragma unroll
             for (int j = 0; j < C::FM; ++j) {
-                const int mrow = lm + j * 16;
+                const int mrow = lm + j * kFrag;
                 const unsigned row_off = mrow < rows_left ? (unsigned)mrow * (unsigned)N * 4u : 0x80000000u;
 #pragma unroll
                 for (int i = 0; i < C::FN; ++i) {
-                    const v4i v = acc[i][j] >> 8;
-                    if (VEC_STORE) {
-                        __builtin_amdgcn_raw_buffer_store_b128((v4u)v, rsrc, row_off + col_off[i], 0, 0);
-                    } else {
-                        // Element e of the four is valid while its column is inside the row.
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            const int ncol = ln + i * 16 + e;
-                            const unsigned off = ncol < cols_left ? row_off + (unsigned)ncol * 4u : 0xC0000000u;
-                            __builtin_amdgcn_raw_buffer_store_b32((unsigned)v[e], rsrc, off, 0, 0);
+                    for (int q = 0; q < 4; ++q) {
+                        const int ncol = ln + i * kFrag + q * 8;
+                        v4i v;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            v[e] = acc[i][j][4 * q + e] >> 8;
+                        if (VEC_STORE) {
+                            const unsigned col_off = ncol + 3 < cols_left ? (unsigned)ncol * 4u : 0x40000000u;
+                            __builtin_amdgcn_raw_buffer_store_b128((v4u)v, rsrc, row_off + col_off, 0, 0);
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                const unsigned col_off = ncol + e < cols_left ? (unsigned)(ncol + e) * 4u : 0x40000000u;
+                                __builtin_amdgcn_raw_buffer_store_b32((unsigned)v[e], rsrc, row_off + col_off, 0, 0);
+                            }
                         }
                     }
                 }
@@ -307,13 +323,12 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
     }
 }
 
-// 256 x 256 tile, four wavefronts of 128 x 128, one workgroup per CU: the large-shape
-// configuration (nibble widening is amortised over the largest wave tile the 512-entry
-// register file holds).
-using CfgLarge = TileConfig<2, 2, 8, 8, 4, 1>;
+// 256 x 256 tile, eight wavefronts of 128 (m) x 64 (n), one workgroup per CU, two
+// wavefronts per SIMD: the large-shape configuration.
+using CfgLarge = TileConfig<2, 4, 4, 2, 4, 1>;
 // 128 x 128 tile, four wavefronts of 64 x 64, two workgroups per CU: mid-sized shapes
 // whose 256 x 256 tile count would leave CUs idle.
-using CfgMedium = TileConfig<2, 2, 4, 4, 4, 2>;
+using CfgMedium = TileConfig<2, 2, 2, 2, 4, 2>;
 
 template <class C>
 hipError_t set_lds_limit()
@@ -338,7 +353,7 @@ hipError_t launch_cfg(const void *a, const void *b, void *c, int m, int n, int k
     long grid = (long)dev.cu_count * C::OCC;
     if (grid > total)
         grid = total;
-    // The epilogue addresses a tile's slab of C with 32-bit byte offsets.
+    // The epilogue addresses a tile's slab of C with 32-bit byte offsets below 2^30.
     if ((size_t)C::BM * (size_t)n * 4u > 0x40000000ull)
         return hipErrorInvalidValue;
     if (n % 4 == 0)
@@ -355,7 +370,7 @@ hipError_t launch_cfg(const void *a, const void *b, void *c, int m, int n, int k
 bool mfma_supports(int m, int n, int k)
 {
     // K <= 131071 keeps 256 * (sum of products) inside int32; one LDS row per stage is
-    // 128 nibbles; a row's byte offset inside a tile must fit 32 bits.
+    // 128 nibbles.
     return m >= 1 && n >= 1 && k >= kStageK && k % kStageK == 0 && k <= 131071 - 127;
 }
 
