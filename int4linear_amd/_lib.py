@@ -6,10 +6,13 @@ symbols raises, and every compute call needs a gfx950 device.
 from __future__ import annotations
 
 import ctypes
+import os
 from ctypes import c_char_p, c_int, c_void_p
 from pathlib import Path
 
-LIB_PATH = Path(__file__).resolve().parent / "lib" / "libint4linear.so"
+# INT4LINEAR_LIBRARY overrides the in-tree location (e.g. to try a differently built copy).
+LIB_PATH = Path(os.environ.get("INT4LINEAR_LIBRARY") or
+                Path(__file__).resolve().parent / "lib" / "libint4linear.so")
 
 # (name, restype, argtypes) for every extern "C" symbol of include/int4linear.h.
 C_ABI = [

@@ -26,7 +26,7 @@ CXX_SOURCES = ["packer_host.cpp"]
 HIP_FLAGS = [
     "--offload-arch=gfx950",
     "-O3",
-    "-std=c++17",
+    "-std=c++20",
     "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
@@ -65,7 +65,7 @@ def build_library(verbose: bool = False, save_temps: bool = False) -> Path:
         jobs.append((cmd, obj))
     for src in CXX_SOURCES:
         obj = OBJ_DIR / (src + ".o")
-        jobs.append(([hipcc, "-O3", "-std=c++17", "-fPIC", "-c", str(CSRC / src), "-o", str(obj)], obj))
+        jobs.append(([hipcc, "-O3", "-std=c++20", "-fPIC", "-c", str(CSRC / src), "-o", str(obj)], obj))
     if verbose:
         for cmd, _ in jobs:
             print(" ".join(cmd))

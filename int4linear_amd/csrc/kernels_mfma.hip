@@ -16,13 +16,17 @@
 //   HBM/L2 --global_load_lds_dwordx4 (16 B per lane, straight into LDS)--> NSTAGE-deep ring
 //   LDS    --ds_read_b128 (bank-conflict-free through a 16-byte-chunk XOR swizzle)--> VGPRs
 //   VGPRs  --3 VALU ops per packed dword--> int8 operands --MFMA--> int32 accumulators
-//   accumulators --buffer_store_dwordx4 (W is the MFMA A operand, so each quad of a
-//                 lane's accumulators is four consecutive n)--> C
+//   accumulators --buffer_store_dword (X is the MFMA A operand, so the 32 lanes of a
+//                 half-wave hold 32 consecutive n: every store writes whole 128-byte
+//                 row segments), non-temporal--> C
 // Two wavefronts share each SIMD: while one widens nibbles on the VALU the other keeps
 // the matrix pipe busy.  The kernel is persistent: gridDim.x workgroups walk a list of
 // tiles, and the load ring runs NSTAGE-1 stages ahead of the math ACROSS tile
 // boundaries, so the next tile's first stages are in flight while this tile stores C.
 #include "kernels.h"
+
+#include <type_traits>
+#include <utility>
 
 namespace int4linear {
 
@@ -59,6 +63,13 @@ __device__ __forceinline__ int opaque(int v)
     return v;
 }
 
+// Marks a value as used (and possibly changed) at this point of the program.
+__device__ __forceinline__ void keep(v4i &v) { asm volatile("" : "+v"(v)); }
+
+#ifndef I4L_STORE_AUX
+#define I4L_STORE_AUX 2  // nt: C is written once and not read back by this kernel
+#endif
+
 constexpr int kStageK = 128;                 // nibbles of K per pipeline stage
 constexpr int kRowBytes = kStageK / 2;       // bytes per LDS row (64)
 constexpr int kChunkRows = 16;               // rows moved by one 64-lane 16-byte load
@@ -83,9 +94,9 @@ struct TileConfig {
     static constexpr int X_CH = X_CHUNKS / NWAVES;             // of which from X
     static constexpr int STAGE_BYTES = (BM + BN) * kRowBytes;
     static constexpr int LDS_BYTES = STAGE_BYTES * NSTAGE;
-    static constexpr int STORES = FM * FN * 4;  // dwordx4 stores per lane per tile
+    static constexpr int STORES = FM * FN * 16;  // dword stores per lane per tile
     static_assert(X_CHUNKS % NWAVES == 0 && W_CHUNKS % NWAVES == 0, "chunks must split evenly");
-    static_assert((NSTAGE - 2) * CH + STORES <= 63, "vmcnt is six bits");
+    static_assert(NSTAGE >= 4 && CH <= 63, "vmcnt is six bits");
 };
 
 // Which 16-byte slot of its 64-byte LDS row holds logical chunk c of row r:  c ^ swz(r),
@@ -116,7 +127,7 @@ __device__ __forceinline__ void tile_coords(int v, int total, int tiles_m, int t
     tn = in_group / gsz;
 }
 
-template <class C, bool VEC_STORE>
+template <class C>
 __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
     const uint8_t *__restrict__ X, const uint8_t *__restrict__ W, int32_t *__restrict__ Y,
     int M, int N, int K, int tiles_m, int tiles_n)
@@ -164,16 +175,17 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
         wptr = W + (size_t)n0 * rowbytes;
     };
 
-    auto ld_issue = [&]() {
+    // One stage = CH loads per wave (ld_chunk) followed by the cursor advance.
+    auto ld_chunk = [&](int c) {
         const int buf = issued % C::NSTAGE;
         const unsigned dst = lds_base + buf * C::STAGE_BYTES;
-#pragma unroll
-        for (int c = 0; c < C::CH; ++c) {
-            const bool is_x = c < C::X_CH;
-            const int ci = (is_x ? c : c - C::X_CH) * C::NWAVES + wave;
-            dma16(is_x ? xptr : wptr, voff[c],
-                  dst + (is_x ? 0 : C::BM * kRowBytes) + ci * kChunkBytes);
-        }
+        const bool is_x = c < C::X_CH;
+        const int ci = (is_x ? c : c - C::X_CH) * C::NWAVES + wave;
+#ifndef I4L_EXP_NODMA
+        dma16(is_x ? xptr : wptr, voff[c], dst + (is_x ? 0 : C::BM * kRowBytes) + ci * kChunkBytes);
+#endif
+    };
+    auto ld_advance = [&]() {
         ++issued;
         ++ld_k;
         xptr += kRowBytes;
@@ -184,6 +196,12 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
             if (ld_it < my_tiles)
                 ld_setup_tile(ld_it);
         }
+    };
+    auto ld_issue = [&]() {
+#pragma unroll
+        for (int c = 0; c < C::CH; ++c)
+            ld_chunk(c);
+        ld_advance();
     };
 
     ld_setup_tile(0);
@@ -206,35 +224,151 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
         rd_off[h] = (unsigned)fr * kRowBytes + (unsigned)(((2 * h + fg) ^ fsw) * 16);
     const unsigned x_rd = (unsigned)(wm * C::FM * kFrag * kRowBytes);
     const unsigned w_rd = (unsigned)(C::BM * kRowBytes + wn * C::FN * kFrag * kRowBytes);
-    const int himask = (int)0xF0F0F0F0u;
+    int himask;  // kept in a scalar register: a VALU source operand that costs nothing
+    asm volatile("s_mov_b32 %0, 0xf0f0f0f0" : "=s"(himask));
 
+    // The math is software-pipelined in units of half a stage.  Unit u = (stage, half h)
+    // owns FN W fragments and FM X fragments; step j of a unit issues the 2*FN MFMAs of X
+    // fragment j.  Two wavefronts share a SIMD and run in lockstep between barriers, so a
+    // wave that widened all its nibbles first and multiplied afterwards would leave the
+    // matrix pipe idle while BOTH waves widen.  Instead every MFMA is followed by a few
+    // of the VALU ops that prepare later operands:
+    //   step (u, j) widens X fragment j+1 (or fragment 0 of unit u+1) and, for j >= 1,
+    //   a third of unit u+1's W fragments; step (u, 0) issues the LDS reads of unit u+1.
+    // __builtin_amdgcn_sched_barrier(0) after each slot pins that order.
     v16i acc[C::FN][C::FM];
+    v4i pk_w[2][C::FN], pk_x[2][C::FM];  // packed fragments, by unit parity (= half)
+    v4i wlo[2][C::FN], whi[2][C::FN];    // widened W, by unit parity
+    v4i xlo[2], xhi[2];                  // widened X fragment, by step parity
     int cur_it = 0, kk = 0;
+    static_assert(C::FM % 2 == 0, "step parity must line up across units");
+
+    // One 16-byte LDS read per fragment of half h of stage st.
+    auto read_unit = [&](int st, int h, v4i (&w)[C::FN], v4i (&x)[C::FM]) {
+        const uint8_t *stage = lds + (st % C::NSTAGE) * C::STAGE_BYTES;
+#ifndef I4L_EXP_NOLDS
+#pragma unroll
+        for (int i = 0; i < C::FN; ++i)
+            w[i] = *(const v4i *)(stage + w_rd + rd_off[h] + i * kFrag * kRowBytes);
+#pragma unroll
+        for (int j = 0; j < C::FM; ++j)
+            x[j] = *(const v4i *)(stage + x_rd + rd_off[h] + j * kFrag * kRowBytes);
+#else
+        for (int i = 0; i < C::FN; ++i) keep(w[i]);
+        for (int j = 0; j < C::FM; ++j) keep(x[j]);
+#endif
+    };
+
+    // Op k (0..11) of widening one packed fragment: per dword d = k/3 a shift, its mask
+    // (even-k nibbles) and the mask of the unshifted word (odd-k nibbles).
+    auto widen_op = [&](int k, const v4i &p, v4i &lo, v4i &hi) {
+#ifdef I4L_EXP_NOVALU
+        if (k == 0) { lo = p; hi = p; }
+        return;
+#endif
+        const int d = k / 3;
+        switch (k % 3) {
+        case 0:
+            lo[d] = p[d] << 4;
+            break;
+        case 1:
+            lo[d] = lo[d] & himask;
+            break;
+        default:
+            hi[d] = p[d] & himask;
+            break;
+        }
+    };
+
+    constexpr int kSlots = 2 * C::FN;             // MFMAs per step
+    constexpr int kWOps = 12 * C::FN;             // VALU ops to widen one unit's W
+    constexpr int kWPerStep = (kWOps + C::FM - 2) / (C::FM - 1);  // spread over steps 1..FM-1
+
+    // Step j of the unit with parity h.  `next_x` is the packed X fragment widened during
+    // this step into step parity (j+1)%2.  `extra(slot)` is further work placed behind the
+    // MFMA of that slot; when it contains branches, `pin` keeps this slot's VALU results
+    // from being moved past them.
+    auto step = [&](auto h_tag, auto j_tag, const v4i &next_x, auto &&extra, bool pin) {
+        constexpr int h = decltype(h_tag)::value;
+        constexpr int j = decltype(j_tag)::value;
+        constexpr int w_begin = j == 0 ? 0 : (j - 1) * kWPerStep;
+        constexpr int w_end = j == 0 ? 0 : (j * kWPerStep < kWOps ? j * kWPerStep : kWOps);
+        constexpr int n_ops = 12 + (w_end - w_begin);
+        [&]<int... SLOT>(std::integer_sequence<int, SLOT...>) {
+            ([&] {
+                constexpr int slot = SLOT;
+                constexpr int i = slot % C::FN;
+                if (slot < C::FN)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(xlo[j % 2], wlo[h][i], acc[i][j], 0, 0, 0);
+                else
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(xhi[j % 2], whi[h][i], acc[i][j], 0, 0, 0);
+                constexpr int op0 = slot * n_ops / kSlots, op1 = (slot + 1) * n_ops / kSlots;
+#pragma unroll
+                for (int op = op0; op < op1; ++op) {
+                    if (op < 12) {
+                        widen_op(op, next_x, xlo[(j + 1) % 2], xhi[(j + 1) % 2]);
+                    } else {
+                        const int wop = w_begin + op - 12;
+                        widen_op(wop % 12, pk_w[1 - h][wop / 12], wlo[1 - h][wop / 12], whi[1 - h][wop / 12]);
+                    }
+                }
+                if (pin) {
+                    keep(xlo[(j + 1) % 2]);
+                    keep(xhi[(j + 1) % 2]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                extra(std::integral_constant<int, slot>{});
+                __builtin_amdgcn_sched_barrier(0);
+            }(), ...);
+        }(std::make_integer_sequence<int, kSlots>{});
+    };
+    auto nothing = [](auto) {};
+
+    // Steps 1..FM-1 of the unit with parity h, then the pins that keep the operands
+    // widened for the next unit (first used after a barrier) inside the MFMA shadow.
+    auto unit_tail = [&](auto h_tag) {
+        constexpr int h = decltype(h_tag)::value;
+        [&]<int... J>(std::integer_sequence<int, J...>) {
+            (step(h_tag, std::integral_constant<int, J + 1>{},
+                  J + 2 < C::FM ? pk_x[h][(J + 2) % C::FM] : pk_x[1 - h][0], nothing, false), ...);
+        }(std::make_integer_sequence<int, C::FM - 1>{});
+#pragma unroll
+        for (int i = 0; i < C::FN; ++i) {
+            keep(wlo[1 - h][i]);
+            keep(whi[1 - h][i]);
+        }
+        keep(xlo[0]);
+        keep(xhi[0]);
+    };
+
+    // Stage 0 must have landed before the first read.
+    if (issued >= C::NSTAGE - 1)
+        __builtin_amdgcn_s_waitcnt(I4L_VMCNT((C::NSTAGE - 2) * C::CH));
+    else
+        __builtin_amdgcn_s_waitcnt(I4L_VMCNT(0));
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    // Pipeline fill: unit (0, 0) read, its W and its X fragment 0 widened.
+    read_unit(0, 0, pk_w[0], pk_x[0]);
+#pragma unroll
+    for (int i = 0; i < C::FN; ++i)
+#pragma unroll
+        for (int op = 0; op < 12; ++op)
+            widen_op(op, pk_w[0][i], wlo[0][i], whi[0][i]);
+#pragma unroll
+    for (int op = 0; op < 12; ++op)
+        widen_op(op, pk_x[0][0], xlo[0], xhi[0]);
+
+    // A wave must not go long without issuing an MFMA: its SIMD partner runs the same
+    // code at the same time, so whatever sits between two MFMAs is matrix-pipe idle time
+    // once it exceeds one MFMA.  The per-stage housekeeping (load wait, barrier, LDS
+    // reads, the CH direct-to-LDS loads, the load cursor) is therefore spread over the
+    // slots of each unit's first step, one piece behind each MFMA.
+    constexpr int kDmaSlots = kSlots - 1;
+    constexpr int kDmaPerSlot = (C::CH + kDmaSlots - 1) / kDmaSlots;
 
 #pragma unroll 1
     for (int gs = 0; gs < total_stages; ++gs) {
-        // Wait until this wave's loads of stage gs have landed.  Outstanding VMEM ops
-        // complete in order; `ahead` stages were issued after stage gs, and the C stores
-        // of the previous tile sit behind the loads of that tile's successor stages.
-        const int ahead = issued - 1 - gs;
-        if (ahead >= C::NSTAGE - 2) {
-            if (cur_it > 0 && kk < C::NSTAGE - 1) {
-                constexpr int stores = VEC_STORE ? C::STORES : 4 * C::STORES;
-                constexpr int with_stores = (C::NSTAGE - 2) * C::CH + stores;
-                __builtin_amdgcn_s_waitcnt(I4L_VMCNT(with_stores < 63 ? with_stores : 63));
-            } else {
-                __builtin_amdgcn_s_waitcnt(I4L_VMCNT((C::NSTAGE - 2) * C::CH));
-            }
-        } else {
-            __builtin_amdgcn_s_waitcnt(I4L_VMCNT(0));
-        }
-        __builtin_amdgcn_s_barrier();
-        asm volatile("" ::: "memory");
-
-        // Refill the buffer every wave finished reading before the barrier.
-        if (issued < total_stages)
-            ld_issue();
-
         if (kk == 0) {
 #pragma unroll
             for (int i = 0; i < C::FN; ++i)
@@ -245,36 +379,63 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
                         acc[i][j][t] = 0;
         }
 
-        const uint8_t *stage = lds + (gs % C::NSTAGE) * C::STAGE_BYTES;
+        // ---- first half; its first slot issues the LDS reads of the second half
+        step(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, pk_x[0][1 % C::FM],
+             [&](auto slot_tag) {
+                 if constexpr (decltype(slot_tag)::value == 0)
+                     read_unit(gs, 1, pk_w[1], pk_x[1]);
+             },
+             false);
+        unit_tail(std::integral_constant<int, 0>{});
+
+        // ---- second half; its first step makes stage gs+1 readable, refills the buffer
+        //      of stage gs-1 and issues the LDS reads of stage gs+1's first half
+        const bool refill = issued < total_stages;
+        step(std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{}, pk_x[1][1 % C::FM],
+             [&](auto slot_tag) {
+                 constexpr int slot = decltype(slot_tag)::value;
+                 if constexpr (slot == 0) {
+                     // This wave's loads of stage gs+1 must have landed, then every wave's.
+                     // Outstanding VMEM ops complete in order; normally one younger stage is
+                     // in flight behind them, and for the two stages after a tile end the C
+                     // stores of that tile sit behind them as well.
+                     const int ahead = issued - 2 - gs;  // stages issued after stage gs+1
+#ifndef I4L_EXP_NOWAIT
+                     if (ahead >= 1) {
+                         if (cur_it > 0 && kk < 2) {
+                             constexpr int with_stores = C::CH + C::STORES;
+                             __builtin_amdgcn_s_waitcnt(I4L_VMCNT(with_stores < 63 ? with_stores : 63));
+                         } else {
+                             __builtin_amdgcn_s_waitcnt(I4L_VMCNT(C::CH));
+                         }
+                     } else {
+                         __builtin_amdgcn_s_waitcnt(I4L_VMCNT(0));
+                     }
+#endif
+#ifndef I4L_EXP_NOBARRIER
+                     __builtin_amdgcn_s_barrier();
+#endif
+                     asm volatile("" ::: "memory");
+                     // (past the last stage this reads a stale buffer whose contents never
+                     // reach a stored tile; unconditional keeps the LDS wait counts exact)
+                     read_unit(gs + 1, 0, pk_w[0], pk_x[0]);
+                 } else {
+                     // Every wave is past its reads of stage gs-1: refill that buffer.
+                     if (refill) {
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            // W fragments of this half are widened once and stay live; X fragments
-            // stream through.
-            v4i wlo[C::FN], whi[C::FN];
-#pragma unroll
-            for (int i = 0; i < C::FN; ++i) {
-                const v4i ww = *(const v4i *)(stage + w_rd + rd_off[h] + i * kFrag * kRowBytes);
-                wlo[i] = (ww << 4) & himask;  // even-k nibbles
-                whi[i] = ww & himask;         // odd-k nibbles
-            }
-#pragma unroll
-            for (int j = 0; j < C::FM; ++j) {
-                const v4i xw = *(const v4i *)(stage + x_rd + rd_off[h] + j * kFrag * kRowBytes);
-                const v4i xlo = (xw << 4) & himask;
-                const v4i xhi = xw & himask;
-#pragma unroll
-                for (int i = 0; i < C::FN; ++i)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wlo[i], xlo, acc[i][j], 0, 0, 0);
-#pragma unroll
-                for (int i = 0; i < C::FN; ++i)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(whi[i], xhi, acc[i][j], 0, 0, 0);
-            }
-        }
+                         for (int c = (slot - 1) * kDmaPerSlot; c < slot * kDmaPerSlot && c < C::CH; ++c)
+                             ld_chunk(c);
+                         if (slot == kSlots - 1)
+                             ld_advance();
+                     }
+                 }
+             },
+             true);
+        unit_tail(std::integral_constant<int, 1>{});
 
         ++kk;
         if (kk == KT) {
-            // ---- store the tile.  Accumulator t of MFMA tile (i, j) belongs to
-            //      n = 32*i + 8*(t/4) + 4*(lane/32) + t%4,  m = 32*j + lane%32.
+            // ---- store the tile
             int tm, tn;
             tile_coords(bid + cur_it * nblk, total_tiles, tiles_m, tiles_n, tm, tn);
             const int m0 = tm * C::BM, n0 = tn * C::BN;
@@ -286,34 +447,35 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
             const size_t extent = ((slab_rows - 1) * (size_t)N + (size_t)(cols_left < C::BN ? cols_left : C::BN)) * 4u;
             __amdgpu_buffer_rsrc_t rsrc =
                 __builtin_amdgcn_make_buffer_rsrc(ybase, 0, (int)extent, 0x00020000);
+            // X is the MFMA A operand: accumulator t of tile (i, j) belongs to
+            //   m = 32*j + 8*(t/4) + 4*(lane/32) + t%4,  n = 32*i + lane%32,
+            // so one dword store writes two rows of 32 consecutive n (128 B each).
             // Offsets are split into a row part and a column part; a lane outside the
             // matrix gets a part so large that the sum falls outside the descriptor's
             // range and the hardware drops the store.
-            const int lm = opaque(wm * C::FM * kFrag + fr);      // tile-relative m (plus 32*j)
-            const int ln = opaque(wn * C::FN * kFrag + fg * 4);  // tile-relative n (plus 32*i + 8*q)
+            const int lm = opaque(wm * C::FM * kFrag + fg * 4);
+            const int ln = opaque(wn * C::FN * kFrag + fr);
+            const unsigned lm_off = (unsigned)lm * (unsigned)N * 4u;
+            unsigned col_off[C::FN];
+#pragma unroll
+            for (int i = 0; i < C::FN; ++i) {
+                const int ncol = ln + i * kFrag;
+                col_off[i] = ncol < cols_left ? (unsigned)ncol * 4u : 0x40000000u;
+            }
 #pragma unroll
             for (int j = 0; j < C::FM; ++j) {
-                const int mrow = lm + j * kFrag;
-                const unsigned row_off = mrow < rows_left ? (unsigned)mrow * (unsigned)N * 4u : 0x80000000u;
 #pragma unroll
-                for (int i = 0; i < C::FN; ++i) {
+                for (int t = 0; t < 16; ++t) {
+                    const int dm = j * kFrag + 8 * (t / 4) + (t % 4);   // uniform
+                    const unsigned row_off = lm + dm < rows_left ? lm_off + (unsigned)dm * (unsigned)N * 4u : 0x80000000u;
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const int ncol = ln + i * kFrag + q * 8;
-                        v4i v;
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            v[e] = acc[i][j][4 * q + e] >> 8;
-                        if (VEC_STORE) {
-                            const unsigned col_off = ncol + 3 < cols_left ? (unsigned)ncol * 4u : 0x40000000u;
-                            __builtin_amdgcn_raw_buffer_store_b128((v4u)v, rsrc, row_off + col_off, 0, 0);
-                        } else {
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) {
-                                const unsigned col_off = ncol + e < cols_left ? (unsigned)(ncol + e) * 4u : 0x40000000u;
-                                __builtin_amdgcn_raw_buffer_store_b32((unsigned)v[e], rsrc, row_off + col_off, 0, 0);
-                            }
-                        }
+                    for (int i = 0; i < C::FN; ++i) {
+                        const int v = acc[i][j][t] >> 8;
+#ifdef I4L_EXP_NOSTORE
+                        if (v == 0x12345) __builtin_amdgcn_raw_buffer_store_b32((unsigned)v, rsrc, 0, 0, 0);
+                        continue;
+#endif
+                        __builtin_amdgcn_raw_buffer_store_b32((unsigned)v, rsrc, row_off + col_off[i], 0, I4L_STORE_AUX);
                     }
                 }
             }
@@ -333,11 +495,7 @@ using CfgMedium = TileConfig<2, 2, 2, 2, 4, 2>;
 template <class C>
 hipError_t set_lds_limit()
 {
-    hipError_t e = hipFuncSetAttribute((const void *)mfma_gemm_kernel<C, true>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
-    if (e != hipSuccess)
-        return e;
-    return hipFuncSetAttribute((const void *)mfma_gemm_kernel<C, false>,
+    return hipFuncSetAttribute((const void *)mfma_gemm_kernel<C>,
                                hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
 }
 
@@ -356,12 +514,8 @@ hipError_t launch_cfg(const void *a, const void *b, void *c, int m, int n, int k
     // The epilogue addresses a tile's slab of C with 32-bit byte offsets below 2^30.
     if ((size_t)C::BM * (size_t)n * 4u > 0x40000000ull)
         return hipErrorInvalidValue;
-    if (n % 4 == 0)
-        mfma_gemm_kernel<C, true><<<(unsigned)grid, C::THREADS, C::LDS_BYTES, stream>>>(
-            (const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k, tiles_m, tiles_n);
-    else
-        mfma_gemm_kernel<C, false><<<(unsigned)grid, C::THREADS, C::LDS_BYTES, stream>>>(
-            (const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k, tiles_m, tiles_n);
+    mfma_gemm_kernel<C><<<(unsigned)grid, C::THREADS, C::LDS_BYTES, stream>>>(
+        (const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k, tiles_m, tiles_n);
     return hipGetLastError();
 }
 
