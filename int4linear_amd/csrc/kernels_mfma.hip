@@ -236,6 +236,21 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
     //   step (u, j) widens X fragment j+1 (or fragment 0 of unit u+1) and, for j >= 1,
     //   a third of unit u+1's W fragments; step (u, 0) issues the LDS reads of unit u+1.
     // __builtin_amdgcn_sched_barrier(0) after each slot pins that order.
+#ifdef I4L_EXP_TRACE
+    long long *trace = (long long *)(lds + C::LDS_BYTES);
+    int trace_n = 0;
+    const bool tracer = (bid == I4L_EXP_TRACE) && (threadIdx.x == I4L_EXP_TRACE_WAVE * 64);
+#ifdef I4L_EXP_TRACE_STEPS
+#define I4L_STAMP() do {} while (0)
+#define I4L_STAMP2() do { if (tracer && trace_n < 3900) { trace[trace_n++] = __builtin_readcyclecounter(); } } while (0)
+#else
+#define I4L_STAMP() do { if (tracer && trace_n < 3900) { trace[trace_n++] = __builtin_readcyclecounter(); } } while (0)
+#define I4L_STAMP2() do {} while (0)
+#endif
+#else
+#define I4L_STAMP2() do {} while (0)
+#define I4L_STAMP() do {} while (0)
+#endif
     v16i acc[C::FN][C::FM];
     v4i pk_w[2][C::FN], pk_x[2][C::FM];  // packed fragments, by unit parity (= half)
     v4i wlo[2][C::FN], whi[2][C::FN];    // widened W, by unit parity
@@ -243,20 +258,23 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
     int cur_it = 0, kk = 0;
     static_assert(C::FM % 2 == 0, "step parity must line up across units");
 
-    // One 16-byte LDS read per fragment of half h of stage st.
-    auto read_unit = [&](int st, int h, v4i (&w)[C::FN], v4i (&x)[C::FM]) {
+    // One 16-byte LDS read per fragment of half h of stage st.  A unit's reads come in
+    // kReadParts parts so that they can be spread over several steps: part 0 is the W
+    // fragments, the others split the X fragments evenly.
+    constexpr int kReadParts = 3;
+    constexpr int kXPerPart = C::FM / (kReadParts - 1);
+    static_assert(kXPerPart * (kReadParts - 1) == C::FM, "X fragments must split evenly");
+    auto read_part = [&](int st, int h, int part, v4i (&w)[C::FN], v4i (&x)[C::FM]) {
         const uint8_t *stage = lds + (st % C::NSTAGE) * C::STAGE_BYTES;
-#ifndef I4L_EXP_NOLDS
+        if (part == 0) {
 #pragma unroll
-        for (int i = 0; i < C::FN; ++i)
-            w[i] = *(const v4i *)(stage + w_rd + rd_off[h] + i * kFrag * kRowBytes);
+            for (int i = 0; i < C::FN; ++i)
+                w[i] = *(const v4i *)(stage + w_rd + rd_off[h] + i * kFrag * kRowBytes);
+        } else {
 #pragma unroll
-        for (int j = 0; j < C::FM; ++j)
-            x[j] = *(const v4i *)(stage + x_rd + rd_off[h] + j * kFrag * kRowBytes);
-#else
-        for (int i = 0; i < C::FN; ++i) keep(w[i]);
-        for (int j = 0; j < C::FM; ++j) keep(x[j]);
-#endif
+            for (int j = (part - 1) * kXPerPart; j < part * kXPerPart; ++j)
+                x[j] = *(const v4i *)(stage + x_rd + rd_off[h] + j * kFrag * kRowBytes);
+        }
     };
 
     // Op k (0..11) of widening one packed fragment: per dword d = k/3 a shift, its mask
@@ -285,10 +303,9 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
     constexpr int kWPerStep = (kWOps + C::FM - 2) / (C::FM - 1);  // spread over steps 1..FM-1
 
     // Step j of the unit with parity h.  `next_x` is the packed X fragment widened during
-    // this step into step parity (j+1)%2.  `extra(slot)` is further work placed behind the
-    // MFMA of that slot; when it contains branches, `pin` keeps this slot's VALU results
-    // from being moved past them.
-    auto step = [&](auto h_tag, auto j_tag, const v4i &next_x, auto &&extra, bool pin) {
+    // this step into step parity (j+1)%2.  `hook(j, slot)` is housekeeping placed behind
+    // the MFMA of that slot; it may branch, so the slot's VALU results are pinned first.
+    auto step = [&](auto h_tag, auto j_tag, const v4i &next_x, auto &&hook) {
         constexpr int h = decltype(h_tag)::value;
         constexpr int j = decltype(j_tag)::value;
         constexpr int w_begin = j == 0 ? 0 : (j - 1) * kWPerStep;
@@ -312,33 +329,29 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
                         widen_op(wop % 12, pk_w[1 - h][wop / 12], wlo[1 - h][wop / 12], whi[1 - h][wop / 12]);
                     }
                 }
-                if (pin) {
-                    keep(xlo[(j + 1) % 2]);
-                    keep(xhi[(j + 1) % 2]);
-                }
+                keep(xlo[(j + 1) % 2]);
+                keep(xhi[(j + 1) % 2]);
                 __builtin_amdgcn_sched_barrier(0);
-                extra(std::integral_constant<int, slot>{});
+                hook(j_tag, std::integral_constant<int, slot>{});
                 __builtin_amdgcn_sched_barrier(0);
             }(), ...);
         }(std::make_integer_sequence<int, kSlots>{});
     };
-    auto nothing = [](auto) {};
 
-    // Steps 1..FM-1 of the unit with parity h, then the pins that keep the operands
-    // widened for the next unit (first used after a barrier) inside the MFMA shadow.
-    auto unit_tail = [&](auto h_tag) {
+    auto stamp2 = [&] { I4L_STAMP2(); };
+    // All steps of the unit with parity h, then the pins that keep the operands widened
+    // for the next unit inside this unit's MFMA shadow.
+    auto unit = [&](auto h_tag, auto &&hook) {
         constexpr int h = decltype(h_tag)::value;
         [&]<int... J>(std::integer_sequence<int, J...>) {
-            (step(h_tag, std::integral_constant<int, J + 1>{},
-                  J + 2 < C::FM ? pk_x[h][(J + 2) % C::FM] : pk_x[1 - h][0], nothing, false), ...);
-        }(std::make_integer_sequence<int, C::FM - 1>{});
+            ((step(h_tag, std::integral_constant<int, J>{},
+                   J + 1 < C::FM ? pk_x[h][(J + 1) % C::FM] : pk_x[1 - h][0], hook), stamp2()), ...);
+        }(std::make_integer_sequence<int, C::FM>{});
 #pragma unroll
         for (int i = 0; i < C::FN; ++i) {
             keep(wlo[1 - h][i]);
             keep(whi[1 - h][i]);
         }
-        keep(xlo[0]);
-        keep(xhi[0]);
     };
 
     // Stage 0 must have landed before the first read.
@@ -349,7 +362,9 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     // Pipeline fill: unit (0, 0) read, its W and its X fragment 0 widened.
-    read_unit(0, 0, pk_w[0], pk_x[0]);
+#pragma unroll
+    for (int part = 0; part < kReadParts; ++part)
+        read_part(0, 0, part, pk_w[0], pk_x[0]);
 #pragma unroll
     for (int i = 0; i < C::FN; ++i)
 #pragma unroll
@@ -359,16 +374,46 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
     for (int op = 0; op < 12; ++op)
         widen_op(op, pk_x[0][0], xlo[0], xhi[0]);
 
-    // A wave must not go long without issuing an MFMA: its SIMD partner runs the same
-    // code at the same time, so whatever sits between two MFMAs is matrix-pipe idle time
-    // once it exceeds one MFMA.  The per-stage housekeeping (load wait, barrier, LDS
-    // reads, the CH direct-to-LDS loads, the load cursor) is therefore spread over the
-    // slots of each unit's first step, one piece behind each MFMA.
-    constexpr int kDmaSlots = kSlots - 1;
-    constexpr int kDmaPerSlot = (C::CH + kDmaSlots - 1) / kDmaSlots;
+    // Housekeeping is spread thinly behind the MFMAs, for two reasons.  A wave must not
+    // go long without issuing an MFMA: its SIMD partner runs the same code at the same
+    // time, so whatever sits between two MFMAs is matrix-pipe idle time once it exceeds
+    // one MFMA.  And the eight waves of a workgroup run in step between barriers, so work
+    // that all of them issue at the same point (32 direct-to-LDS loads, 48 LDS reads)
+    // queues up in the memory pipeline and blocks the waves behind it.  Hence:
+    //   * the LDS reads of the next unit go out in kReadParts parts, evenly spaced over
+    //     the unit's FM * kSlots slot positions;
+    //   * the CH loads of stage gs+3 are split between the second half of iteration gs
+    //     (loads 0..CH/2-1) and the first half of iteration gs+1 (the rest); inside a half
+    //     they are evenly spaced and odd waves go one place after even waves, so at any
+    //     position at most half the waves issue one load;
+    //   * the load cursor advances at the last position of the first half.
+    // All loads of stage gs+3 are still issued between the barriers of iterations gs and
+    // gs+1, in order, which is all the wait counts below rely on.
+    constexpr int kPositions = C::FM * kSlots;       // slot positions per unit
+    constexpr int kDmaStride = kPositions / C::CH;   // CH/2 loads x 2 wave parities per half
+    static_assert(C::CH % 2 == 0 && kDmaStride >= 1 && kDmaStride * C::CH == kPositions,
+                  "load spreading needs CH places per half");
+    const int wave_par = wave & 1;
+    bool loading = false;  // a stage's loads are partly issued
+    // Housekeeping common to both halves at position (j, slot): `read_st`/`read_h` name the
+    // unit whose fragments are read, `half_pos` is 0 in the second half of an iteration.
+    auto spread = [&](auto j_tag, auto slot_tag, int read_st, int read_h, int half_pos) {
+        constexpr int pos = decltype(j_tag)::value * kSlots + decltype(slot_tag)::value;
+#pragma unroll
+        for (int part = 0; part < kReadParts; ++part)
+            if (pos == part * kPositions / kReadParts + 1)
+                read_part(read_st, read_h, part, pk_w[read_h], pk_x[read_h]);
+        constexpr int off = kDmaStride / 2;
+        if constexpr (pos >= off && (pos - off) % kDmaStride == 0) {
+            constexpr int idx = (pos - off) / kDmaStride;  // 0 .. CH-1
+            if (loading && wave_par == idx % 2)
+                ld_chunk(half_pos * (C::CH / 2) + idx / 2);
+        }
+    };
 
 #pragma unroll 1
     for (int gs = 0; gs < total_stages; ++gs) {
+        I4L_STAMP2();
         if (kk == 0) {
 #pragma unroll
             for (int i = 0; i < C::FN; ++i)
@@ -379,59 +424,55 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
                         acc[i][j][t] = 0;
         }
 
-        // ---- first half; its first slot issues the LDS reads of the second half
-        step(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, pk_x[0][1 % C::FM],
-             [&](auto slot_tag) {
-                 if constexpr (decltype(slot_tag)::value == 0)
-                     read_unit(gs, 1, pk_w[1], pk_x[1]);
-             },
-             false);
-        unit_tail(std::integral_constant<int, 0>{});
+        // ---- first half: reads the second half of this stage, finishes the loads begun
+        //      in the previous iteration
+        unit(std::integral_constant<int, 0>{}, [&](auto j_tag, auto slot_tag) {
+            constexpr int j = decltype(j_tag)::value;
+            constexpr int slot = decltype(slot_tag)::value;
+            spread(j_tag, slot_tag, gs, 1, 1);
+            if constexpr (slot == kSlots - 1 && j == C::FM - 1) {
+                if (loading) {
+                    ld_advance();
+                    loading = false;
+                }
+            }
+        });
 
-        // ---- second half; its first step makes stage gs+1 readable, refills the buffer
-        //      of stage gs-1 and issues the LDS reads of stage gs+1's first half
-        const bool refill = issued < total_stages;
-        step(std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{}, pk_x[1][1 % C::FM],
-             [&](auto slot_tag) {
-                 constexpr int slot = decltype(slot_tag)::value;
-                 if constexpr (slot == 0) {
-                     // This wave's loads of stage gs+1 must have landed, then every wave's.
-                     // Outstanding VMEM ops complete in order; normally one younger stage is
-                     // in flight behind them, and for the two stages after a tile end the C
-                     // stores of that tile sit behind them as well.
-                     const int ahead = issued - 2 - gs;  // stages issued after stage gs+1
+        // ---- second half: makes stage gs+1 readable, reads its first half, begins the
+        //      loads of stage gs+3 into the buffer of stage gs-1
+        unit(std::integral_constant<int, 1>{}, [&](auto j_tag, auto slot_tag) {
+            constexpr int j = decltype(j_tag)::value;
+            constexpr int slot = decltype(slot_tag)::value;
+            if constexpr (slot == 0 && j == 0) {
+                // This wave's loads of stage gs+1 must have landed, then every wave's.
+                // Outstanding VMEM ops complete in order; normally one younger stage is in
+                // flight behind them, and in the first stage after a tile end the C stores
+                // of that tile sit behind them as well.  (One stage later the loads waited
+                // for were themselves issued after those stores, so the stores must be done.)
+                const int ahead = issued - 2 - gs;  // stages issued after stage gs+1
 #ifndef I4L_EXP_NOWAIT
-                     if (ahead >= 1) {
-                         if (cur_it > 0 && kk < 2) {
-                             constexpr int with_stores = C::CH + C::STORES;
-                             __builtin_amdgcn_s_waitcnt(I4L_VMCNT(with_stores < 63 ? with_stores : 63));
-                         } else {
-                             __builtin_amdgcn_s_waitcnt(I4L_VMCNT(C::CH));
-                         }
-                     } else {
-                         __builtin_amdgcn_s_waitcnt(I4L_VMCNT(0));
-                     }
+                if (ahead >= 1) {
+                    if (cur_it > 0 && kk < 1) {
+                        constexpr int with_stores = C::CH + C::STORES;
+                        __builtin_amdgcn_s_waitcnt(I4L_VMCNT(with_stores < 63 ? with_stores : 63));
+                    } else {
+                        __builtin_amdgcn_s_waitcnt(I4L_VMCNT(C::CH));
+                    }
+                } else {
+                    __builtin_amdgcn_s_waitcnt(I4L_VMCNT(0));
+                }
 #endif
 #ifndef I4L_EXP_NOBARRIER
-                     __builtin_amdgcn_s_barrier();
+                __builtin_amdgcn_s_barrier();
 #endif
-                     asm volatile("" ::: "memory");
-                     // (past the last stage this reads a stale buffer whose contents never
-                     // reach a stored tile; unconditional keeps the LDS wait counts exact)
-                     read_unit(gs + 1, 0, pk_w[0], pk_x[0]);
-                 } else {
-                     // Every wave is past its reads of stage gs-1: refill that buffer.
-                     if (refill) {
-#pragma unroll
-                         for (int c = (slot - 1) * kDmaPerSlot; c < slot * kDmaPerSlot && c < C::CH; ++c)
-                             ld_chunk(c);
-                         if (slot == kSlots - 1)
-                             ld_advance();
-                     }
-                 }
-             },
-             true);
-        unit_tail(std::integral_constant<int, 1>{});
+                asm volatile("" ::: "memory");
+                // Every wave is past its reads of stage gs-1: that buffer may be refilled.
+                loading = issued < total_stages;
+            }
+            // (past the last stage the reads fetch a stale buffer whose contents never reach
+            // a stored tile; unconditional reads keep the LDS wait counts exact)
+            spread(j_tag, slot_tag, gs + 1, 0, 0);
+        });
 
         ++kk;
         if (kk == KT) {
@@ -483,6 +524,16 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
             ++cur_it;
         }
     }
+#ifdef I4L_EXP_TRACE
+    I4L_STAMP();
+    __builtin_amdgcn_s_waitcnt(0);
+    if (tracer) {
+        long long *dst = (long long *)Y;
+        dst[0] = trace_n;
+        for (int i = 0; i < trace_n; ++i)
+            dst[1 + i] = trace[i];
+    }
+#endif
 }
 
 // 256 x 256 tile, eight wavefronts of 128 (m) x 64 (n), one workgroup per CU, two
@@ -514,6 +565,12 @@ hipError_t launch_cfg(const void *a, const void *b, void *c, int m, int n, int k
     // The epilogue addresses a tile's slab of C with 32-bit byte offsets below 2^30.
     if ((size_t)C::BM * (size_t)n * 4u > 0x40000000ull)
         return hipErrorInvalidValue;
+#ifdef I4L_EXP_TRACE
+    hipFuncSetAttribute((const void *)mfma_gemm_kernel<C>, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES + 32000);
+    mfma_gemm_kernel<C><<<(unsigned)grid, C::THREADS, C::LDS_BYTES + 32000, stream>>>(
+        (const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k, tiles_m, tiles_n);
+    return hipGetLastError();
+#endif
     mfma_gemm_kernel<C><<<(unsigned)grid, C::THREADS, C::LDS_BYTES, stream>>>(
         (const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k, tiles_m, tiles_n);
     return hipGetLastError();
