@@ -13,11 +13,16 @@
  *   2. the reference's own C++-linkage entry points (linear_vN_launch, pack, unpack)
  *      with the reference's signatures and blocking behaviour, implemented on top of 1.
  *
- * All pointers named *_d are device pointers owned by the caller.  The library makes
- * no device allocation in any entry point declared here.
+ * All pointers named *_d are device pointers owned by the caller.  The only device
+ * memory the library itself allocates is one workspace per device for the FP6 kernel
+ * (see int4linear_workspace_bytes): created on first need, grown when a larger problem
+ * arrives, never larger than the workspace limit, freed by int4linear_release_workspace
+ * or at process exit.  With the limit set to 0 no entry point allocates anything.
  */
 #ifndef INT4LINEAR_H
 #define INT4LINEAR_H
+
+#include <stddef.h>
 
 #ifdef __cplusplus
 extern "C" {
@@ -39,7 +44,10 @@ enum {
     INT4LINEAR_KERNEL_AUTO = 0,   /* shape-based dispatch (what the plain entry uses)    */
     INT4LINEAR_KERNEL_SIMPLE = 1, /* one thread per output, scalar nibble decode; any K%8==0 */
     INT4LINEAR_KERNEL_MFMA = 2,   /* LDS-pipelined v_mfma_i32_16x16x64_i8 kernel; K%128==0 */
-    INT4LINEAR_KERNEL_SKINNY = 3  /* weight-streaming kernel for M <= 64; K%128==0       */
+    INT4LINEAR_KERNEL_SKINNY = 3, /* weight-streaming kernel for M <= 64; K%128==0       */
+    INT4LINEAR_KERNEL_FP6 = 4     /* operands converted to FP6 (E2M3) in a workspace, then
+                                     v_mfma_scale_f32_32x32x64_f8f6f4; exact; K%128==0,
+                                     K < 2^18                                            */
 };
 
 /* One-time set-up for the current HIP device (queries the CU count, raises the
@@ -67,8 +75,19 @@ int int4linear_gemm_s4s4s32_ex(const void *a_packed_d, const void *b_packed_d, v
 int int4linear_pack_s32_to_s4(const int *src_d, int *dst_d, int m, int n, void *stream);
 int int4linear_unpack_s4_to_s32(const int *src_d, int *dst_d, int m, int n, void *stream);
 
+/* Bytes of internal workspace INT4LINEAR_KERNEL_AUTO would use for a shape (0 when the
+ * chosen kernel needs none). */
+size_t int4linear_workspace_bytes(int m, int n, int k);
+
+/* Upper bound for the internal workspace (default 1 GiB).  Shapes that would need more,
+ * and every shape when the limit is 0, run on the kernels that need no workspace. */
+void int4linear_set_workspace_limit(size_t bytes);
+
+/* Frees the current device's internal workspace (it is re-created on next need). */
+int int4linear_release_workspace(void);
+
 /* Name of the kernel INT4LINEAR_KERNEL_AUTO would pick for a shape ("simple", "mfma",
- * "skinny"); never NULL. */
+ * "fp6", "skinny"); never NULL. */
 const char *int4linear_kernel_for_shape(int m, int n, int k);
 
 /* Human-readable text for a status code; never NULL. */

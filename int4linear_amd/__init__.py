@@ -18,7 +18,10 @@ from .api import (  # noqa: F401
     pack,
     pack_device,
     pack_rows,
+    release_workspace,
+    set_workspace_limit,
     unpack,
     unpack_device,
+    workspace_bytes,
 )
 from ._lib import Int4LinearError  # noqa: F401

@@ -7,7 +7,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import c_char_p, c_int, c_void_p
+from ctypes import c_char_p, c_int, c_size_t, c_void_p
 from pathlib import Path
 
 # INT4LINEAR_LIBRARY overrides the in-tree location (e.g. to try a differently built copy).
@@ -22,6 +22,9 @@ C_ABI = [
      [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     ("int4linear_pack_s32_to_s4", c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
     ("int4linear_unpack_s4_to_s32", c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
+    ("int4linear_workspace_bytes", c_size_t, [c_int, c_int, c_int]),
+    ("int4linear_set_workspace_limit", None, [c_size_t]),
+    ("int4linear_release_workspace", c_int, []),
     ("int4linear_kernel_for_shape", c_char_p, [c_int, c_int, c_int]),
     ("int4linear_status_string", c_char_p, [c_int]),
     ("int4linear_last_hip_error", c_int, []),

@@ -14,7 +14,7 @@ import numpy as np
 
 from . import _lib
 
-KERNELS = {"auto": 0, "simple": 1, "mfma": 2, "skinny": 3}
+KERNELS = {"auto": 0, "simple": 1, "mfma": 2, "skinny": 3, "fp6": 4}
 
 
 def _ptr(obj) -> int:
@@ -49,6 +49,19 @@ def gemm_s4s4s32(a_packed_d, b_packed_d, c_d, m: int, n: int, k: int, *, kernel:
     st = lib.int4linear_gemm_s4s4s32_ex(_ptr(a_packed_d), _ptr(b_packed_d), _ptr(c_d), m, n, k,
                                         KERNELS[kernel], ctypes.c_void_p(stream))
     _lib.check(st)
+
+
+def workspace_bytes(m: int, n: int, k: int) -> int:
+    """Internal workspace the automatic dispatch would use for this shape."""
+    return int(_lib.load().int4linear_workspace_bytes(m, n, k))
+
+
+def set_workspace_limit(nbytes: int) -> None:
+    _lib.load().int4linear_set_workspace_limit(nbytes)
+
+
+def release_workspace() -> None:
+    _lib.check(_lib.load().int4linear_release_workspace())
 
 
 def kernel_for_shape(m: int, n: int, k: int) -> str:

@@ -19,7 +19,7 @@ LIB_DIR = PKG_DIR / "lib"
 OBJ_DIR = PKG_DIR / "csrc" / "build"
 LIB_PATH = LIB_DIR / "libint4linear.so"
 
-HIP_SOURCES = ["api.hip", "kernels_simple.hip", "kernels_mfma.hip", "kernels_skinny.hip"]
+HIP_SOURCES = ["api.hip", "kernels_simple.hip", "kernels_mfma.hip", "kernels_fp6.hip", "kernels_skinny.hip"]
 CXX_SOURCES = ["packer_host.cpp"]
 
 # Packed-FP32 VALU forms are switched off for every device compile of this project.

@@ -2,6 +2,7 @@
 #include "../../include/int4linear.h"
 #include "kernels.h"
 
+#include <atomic>
 #include <cstdint>
 #include <cstdio>
 #include <mutex>
@@ -17,7 +18,18 @@ struct PerDevice {
     hipError_t init_error = hipSuccess;
     int status = INT4LINEAR_OK;
     DeviceInfo info;
+    // Workspace of the FP6 path: grown on demand up to g_workspace_limit, kept until
+    // int4linear_release_workspace() or process exit.  `ws_event` marks the end of the
+    // last GEMM that used it, so a call on another stream can wait for it.
+    std::mutex ws_mutex;
+    void *ws = nullptr;
+    size_t ws_bytes = 0;
+    hipEvent_t ws_event = nullptr;
+    hipStream_t ws_stream = nullptr;
+    bool ws_used = false;
 };
+
+std::atomic<size_t> g_workspace_limit{(size_t)1 << 30};
 
 PerDevice g_devices[kMaxDevices];
 thread_local int t_last_hip_error = 0;
@@ -51,6 +63,8 @@ int ensure_init(PerDevice **out)
         pd.info.cu_count = prop.multiProcessorCount;
         pd.info.lds_per_cu = (int)prop.maxSharedMemoryPerMultiProcessor;
         err = mfma_init(pd.info);
+        if (err == hipSuccess)
+            err = fp6_init(pd.info);
         if (err != hipSuccess) {
             pd.init_error = err;
             pd.status = INT4LINEAR_ERR_HIP;
@@ -67,13 +81,72 @@ int ensure_init(PerDevice **out)
 
 bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 
+// The FP6 path pays off once its 256 x 256 tiles can occupy a good part of the device
+// (its converter pass is a fixed cost of about (M + N) * K * 1.25 bytes of HBM traffic).
+bool fp6_worthwhile(int m, int n, int k)
+{
+    const long tiles = (long)((m + 255) / 256) * ((n + 255) / 256);
+    return fp6_supports(m, n, k) && tiles >= 128 &&
+           fp6_workspace_bytes(m, n, k) <= g_workspace_limit.load();
+}
+
 int pick_kernel(int m, int n, int k)
 {
     if (skinny_supports(m, n, k))
         return INT4LINEAR_KERNEL_SKINNY;
+    if (fp6_worthwhile(m, n, k))
+        return INT4LINEAR_KERNEL_FP6;
     if (mfma_supports(m, n, k))
         return INT4LINEAR_KERNEL_MFMA;
     return INT4LINEAR_KERNEL_SIMPLE;
+}
+
+// Runs the FP6 path on the device's internal workspace.  Calls on one stream are ordered
+// by the stream; a call on a different stream than the previous user first waits for
+// that user's GEMM to finish with the workspace.
+int run_fp6(PerDevice *pd, const void *a, const void *b, void *c, int m, int n, int k,
+            hipStream_t stream)
+{
+    const size_t need = fp6_workspace_bytes(m, n, k);
+    if (need > g_workspace_limit.load())
+        return INT4LINEAR_ERR_UNSUPPORTED;
+    std::lock_guard<std::mutex> lock(pd->ws_mutex);
+    hipError_t e;
+    if (!pd->ws_event) {
+        e = hipEventCreateWithFlags(&pd->ws_event, hipEventDisableTiming);
+        if (e != hipSuccess)
+            return fail_hip(e);
+    }
+    if (pd->ws_bytes < need) {
+        if (pd->ws) {
+            e = hipFree(pd->ws);  // waits for the device to be done with it
+            pd->ws = nullptr;
+            pd->ws_bytes = 0;
+            pd->ws_used = false;
+            if (e != hipSuccess)
+                return fail_hip(e);
+        }
+        e = hipMalloc(&pd->ws, need);
+        if (e != hipSuccess) {
+            pd->ws = nullptr;
+            return fail_hip(e);
+        }
+        pd->ws_bytes = need;
+    }
+    if (pd->ws_used && pd->ws_stream != stream) {
+        e = hipStreamWaitEvent(stream, pd->ws_event, 0);
+        if (e != hipSuccess)
+            return fail_hip(e);
+    }
+    e = launch_fp6(a, b, c, m, n, k, pd->ws, pd->info, stream);
+    if (e != hipSuccess)
+        return fail_hip(e);
+    e = hipEventRecord(pd->ws_event, stream);
+    if (e != hipSuccess)
+        return fail_hip(e);
+    pd->ws_stream = stream;
+    pd->ws_used = true;
+    return INT4LINEAR_OK;
 }
 
 int gemm_impl(const void *a, const void *b, void *c, int m, int n, int k, int kernel,
@@ -81,7 +154,7 @@ int gemm_impl(const void *a, const void *b, void *c, int m, int n, int k, int ke
 {
     if (m < 0 || n < 0 || k < 0 || (k % 8) != 0)
         return INT4LINEAR_ERR_SHAPE;
-    if (kernel < INT4LINEAR_KERNEL_AUTO || kernel > INT4LINEAR_KERNEL_SKINNY)
+    if (kernel < INT4LINEAR_KERNEL_AUTO || kernel > INT4LINEAR_KERNEL_FP6)
         return INT4LINEAR_ERR_UNSUPPORTED;
     if (m == 0 || n == 0)
         return INT4LINEAR_OK;
@@ -103,8 +176,19 @@ int gemm_impl(const void *a, const void *b, void *c, int m, int n, int k, int ke
         return e == hipSuccess ? INT4LINEAR_OK : fail_hip(e);
     }
 
-    if (kernel == INT4LINEAR_KERNEL_AUTO)
+    const bool automatic = kernel == INT4LINEAR_KERNEL_AUTO;
+    if (automatic)
         kernel = pick_kernel(m, n, k);
+    if (kernel == INT4LINEAR_KERNEL_FP6) {
+        if (!fp6_supports(m, n, k))
+            return INT4LINEAR_ERR_UNSUPPORTED;
+        const int st6 = run_fp6(pd, a, b, c, m, n, k, stream);
+        // Under automatic dispatch a workspace that cannot be had falls back to the
+        // int8 kernel, which needs none.
+        if (st6 == INT4LINEAR_OK || !automatic)
+            return st6;
+        kernel = INT4LINEAR_KERNEL_MFMA;
+    }
 
     hipError_t e = hipSuccess;
     switch (kernel) {
@@ -197,6 +281,8 @@ const char *int4linear_kernel_for_shape(int m, int n, int k)
     switch (pick_kernel(m, n, k)) {
     case INT4LINEAR_KERNEL_SKINNY:
         return "skinny";
+    case INT4LINEAR_KERNEL_FP6:
+        return "fp6";
     case INT4LINEAR_KERNEL_MFMA:
         return "mfma";
     default:
@@ -227,6 +313,33 @@ const char *int4linear_status_string(int status)
 }
 
 int int4linear_last_hip_error(void) { return t_last_hip_error; }
+
+size_t int4linear_workspace_bytes(int m, int n, int k)
+{
+    if (m < 0 || n < 0 || k < 0 || !fp6_worthwhile(m, n, k) || skinny_supports(m, n, k))
+        return 0;
+    return fp6_workspace_bytes(m, n, k);
+}
+
+void int4linear_set_workspace_limit(size_t bytes) { g_workspace_limit.store(bytes); }
+
+int int4linear_release_workspace(void)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+        return INT4LINEAR_ERR_NO_DEVICE;
+    PerDevice &pd = g_devices[dev];
+    std::lock_guard<std::mutex> lock(pd.ws_mutex);
+    if (pd.ws) {
+        hipError_t e = hipFree(pd.ws);
+        pd.ws = nullptr;
+        pd.ws_bytes = 0;
+        pd.ws_used = false;
+        if (e != hipSuccess)
+            return fail_hip(e);
+    }
+    return INT4LINEAR_OK;
+}
 
 int int4linear_device_cu_count(void)
 {

@@ -21,6 +21,14 @@ hipError_t mfma_init(const DeviceInfo &dev);
 hipError_t launch_mfma(const void *a, const void *b, void *c, int m, int n, int k,
                        const DeviceInfo &dev, hipStream_t stream);
 
+// FP6-MFMA path: converts both operands into a workspace of fp6_workspace_bytes() bytes
+// (256-byte aligned), then runs the GEMM on it.  Requires K % 128 == 0, K < 2^18.
+bool fp6_supports(int m, int n, int k);
+size_t fp6_workspace_bytes(int m, int n, int k);
+hipError_t fp6_init(const DeviceInfo &dev);
+hipError_t launch_fp6(const void *a, const void *b, void *c, int m, int n, int k, void *workspace,
+                      const DeviceInfo &dev, hipStream_t stream);
+
 // Weight-streaming kernel for skinny M.  Requires M <= 64, K % 128 == 0.
 bool skinny_supports(int m, int n, int k);
 hipError_t launch_skinny(const void *a, const void *b, void *c, int m, int n, int k,

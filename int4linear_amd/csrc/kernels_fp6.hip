@@ -1,0 +1,478 @@
+// FP6-MFMA GEMM over signed-int4 operands for gfx950 (CDNA4), exact in int32.
+//
+// CDNA4's matrix cores run the 6-bit float format E2M3 at twice the int8 rate
+// (v_mfma_scale_f32_32x32x64_f8f6f4: 32x32x64 per instruction in the time the int8
+// instruction does 32x32x32), and E2M3 holds every signed 4-bit integer exactly:
+// sign, two exponent bits and three mantissa bits encode n/8 for n = -15..15 as the plain
+// sign-magnitude integer |n| with the sign in bit 5 (subnormals 0..7 are |n| itself, 8 is
+// exponent 1 with mantissa 0).  With both block scales set to 2^3 a product is n*m
+// exactly, the fp32 accumulator holds integers, and fp32 is exact below 2^24, i.e. for
+// K * 64 < 2^24.  The launcher refuses larger K; the result is bit-identical to integer
+// arithmetic (the tests compare it against the CPU oracle).
+//
+// Two kernels:
+//   * fp6_convert_kernel rewrites a packed s4 operand (rows x K/2 bytes) into FP6
+//     "fragment-major" form in a workspace: for every block of 32 rows x 64 k the 24
+//     bytes each of the 64 MFMA lanes feeds to the instruction, stored as 64 x 16 B
+//     followed by 64 x 8 B.  Rows are padded with zeros to a multiple of the 256-row
+//     tile.  HBM-bound: 0.5 B read and 0.75 B written per element.
+//   * fp6_gemm_kernel is a persistent, LDS-pipelined GEMM over those fragments.  Because
+//     the workspace is already in the order lanes consume it, global->LDS is a linear
+//     direct-to-LDS copy, LDS->VGPR is one 16-byte and one 8-byte read per lane per
+//     fragment at consecutive addresses (no swizzle, no bank conflicts), and the main loop
+//     contains no VALU work at all.
+//
+// Order of k inside a fragment is whatever the converter produces; it only has to be the
+// same for both operands, which it is because both go through the same converter.
+#include "kernels.h"
+
+#include <type_traits>
+#include <utility>
+
+namespace int4linear {
+
+namespace {
+
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+#define I4L_LDS(p) ((__attribute__((address_space(3))) void *)(p))
+// s_waitcnt immediate for gfx9: vmcnt[3:0] bits 3:0, vmcnt[5:4] bits 15:14, expcnt bits
+// 6:4, lgkmcnt bits 11:8.  VM only leaves the others at "no wait".
+#define I4L_WAIT_VM(n) ((0x0F70) | ((n) & 0xF) | ((((n) >> 4) & 0x3) << 14))
+#define I4L_WAIT_VM_LGKM0(n) ((0x0070) | ((n) & 0xF) | ((((n) >> 4) & 0x3) << 14))
+
+constexpr int kTileRows = 256;                        // rows of either operand per tile
+constexpr int kFragRows = 32;                         // rows of one MFMA operand
+constexpr int kFragK = 64;                            // k of one MFMA
+constexpr int kFragBytes = 64 * 24;                   // 64 lanes x 192 bits
+constexpr int kFragLoBytes = 64 * 16;                 // the 16-byte parts come first
+constexpr int kStageK = 128;                          // k per pipeline stage
+constexpr int kFragsK = kStageK / kFragK;             // 2
+constexpr int kFragsRows = kTileRows / kFragRows;     // 8
+constexpr int kOperandStageBytes = kFragsK * kFragsRows * kFragBytes;  // 24 KiB
+constexpr int kStageBytes = 2 * kOperandStageBytes;                    // 48 KiB
+constexpr int kStages = 3;
+constexpr int kLdsBytes = kStages * kStageBytes;                       // 144 KiB
+constexpr int kScale = 127 + 3;                       // E8M0 block scale 2^3 for both operands
+
+// ---- converter --------------------------------------------------------------------------
+
+// Four nibble values (one per byte of x, 0..15 meaning 0..7,-8..-1) -> four E2M3 codes
+// (sign << 5 | magnitude), one per byte.
+__device__ __forceinline__ unsigned fp6_codes(unsigned x)
+{
+    const unsigned s = x & 0x08080808u;   // sign bits
+    const unsigned t = s >> 3;            // 1 in negative bytes
+    const unsigned m = t * 15u;           // 0x0F in negative bytes
+    const unsigned mag = (x ^ m) + t;     // 16 - x for negatives, x otherwise
+    return mag | (s << 2);
+}
+
+// Four 6-bit codes, one per byte -> 24 contiguous bits.
+__device__ __forceinline__ unsigned pack_codes(unsigned c)
+{
+    const unsigned t = (c & 0x003F003Fu) | ((c >> 2) & 0x0FC00FC0u);  // 12 bits per half
+    return (t & 0x00000FFFu) | ((t >> 4) & 0x00FFF000u);
+}
+
+// One packed dword (8 nibbles) -> 48 bits of FP6 codes.
+__device__ __forceinline__ unsigned long long fp6_from_dword(unsigned w)
+{
+    const unsigned even = pack_codes(fp6_codes(w & 0x0F0F0F0Fu));
+    const unsigned odd = pack_codes(fp6_codes((w >> 4) & 0x0F0F0F0Fu));
+    return (unsigned long long)even | ((unsigned long long)odd << 24);
+}
+
+// Workspace index of the fragment (tile, stage, k-fragment, row-fragment).
+__device__ __forceinline__ size_t frag_offset(int tile, int stage, int kf, int rf, int stages)
+{
+    return ((((size_t)tile * stages + stage) * kFragsK + kf) * kFragsRows + rf) * (size_t)kFragBytes;
+}
+
+// One workgroup converts 32 rows x 256 k.  Thread t handles row t/8 and the 16-byte chunk
+// t%8 (32 k): eight neighbouring lanes read 128 contiguous bytes of a row and write 128
+// contiguous bytes of a fragment's 16-byte parts.
+__global__ __launch_bounds__(256) void fp6_convert_kernel(const uint8_t *__restrict__ src,
+                                                           uint8_t *__restrict__ ws, int rows,
+                                                           int padded_rows, int k)
+{
+    const int r = threadIdx.x >> 3;
+    const int c = threadIdx.x & 7;
+    const int row = blockIdx.y * kFragRows + r;       // < padded_rows
+    const int kchunk = blockIdx.x * 8 + c;            // 32-k chunk index along the row
+    const int stages = k / kStageK;
+    if (kchunk * 32 >= k)  // K % 256 == 128: the last workgroup of a row is half empty
+        return;
+    v4i w = {0, 0, 0, 0};
+    if (row < rows)
+        w = __builtin_nontemporal_load((const v4i *)(src + (size_t)row * (k >> 1) + (size_t)kchunk * 16));
+    const unsigned long long q0 = fp6_from_dword((unsigned)w[0]);
+    const unsigned long long q1 = fp6_from_dword((unsigned)w[1]);
+    const unsigned long long q2 = fp6_from_dword((unsigned)w[2]);
+    const unsigned long long q3 = fp6_from_dword((unsigned)w[3]);
+    const unsigned long long o0 = q0 | (q1 << 48);
+    const unsigned long long o1 = (q1 >> 16) | (q2 << 32);
+    const unsigned long long o2 = (q2 >> 32) | (q3 << 16);
+
+    const int kfrag = kchunk >> 1;                    // 64-k fragment index along the row
+    const int lane = (kchunk & 1) * 32 + (row & 31);
+    uint8_t *frag = ws + frag_offset(row / kTileRows, kfrag / kFragsK, kfrag % kFragsK,
+                                     (row % kTileRows) / kFragRows, stages);
+    const v4i lo = {(int)o0, (int)(o0 >> 32), (int)o1, (int)(o1 >> 32)};
+    const v2i hi = {(int)o2, (int)(o2 >> 32)};
+    *(v4i *)(frag + lane * 16) = lo;
+    *(v2i *)(frag + kFragLoBytes + lane * 8) = hi;
+}
+
+// ---- GEMM ---------------------------------------------------------------------------------
+
+__device__ __forceinline__ void dma16(const void *sbase, unsigned voff, unsigned lds_addr)
+{
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(voff), "s"(sbase), "s"(lds_addr)
+                 : "memory");
+}
+
+__device__ __forceinline__ int opaque(int v)
+{
+    asm volatile("" : "+v"(v));
+    return v;
+}
+
+// Same XCD-aware grouped tile order as the int8 kernel: workgroup ids go round-robin
+// over 8 XCDs; ids congruent mod 8 get consecutive positions of an 8-tile-row-tall,
+// column-major grouped order so that concurrent tiles of one XCD share operand rows in L2.
+__device__ __forceinline__ void tile_coords(int v, int total, int tiles_m, int tiles_n,
+                                            int &tm, int &tn)
+{
+    constexpr int kXcd = 8, kGroup = 8;
+    const int x = v % kXcd, j = v / kXcd;
+    const int cnt = total / kXcd, rem = total % kXcd;
+    const int q = x * cnt + (x < rem ? x : rem) + j;
+    const int per_group = kGroup * tiles_n;
+    const int group = q / per_group;
+    const int first_m = group * kGroup;
+    const int gsz = (tiles_m - first_m < kGroup) ? (tiles_m - first_m) : kGroup;
+    const int in_group = q % per_group;
+    tm = first_m + in_group % gsz;
+    tn = in_group / gsz;
+}
+
+// WAVES_M x WAVES_N wavefronts per workgroup; each owns FM x FN MFMA tiles of 32x32.
+template <int WAVES_M_, int WAVES_N_, int OCC_>
+struct Fp6Config {
+    static constexpr int WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, OCC = OCC_;
+    static constexpr int NWAVES = WAVES_M * WAVES_N;
+    static constexpr int THREADS = NWAVES * 64;
+    static constexpr int FM = kTileRows / kFragRows / WAVES_M;
+    static constexpr int FN = kTileRows / kFragRows / WAVES_N;
+    static constexpr int CHUNKS = kStageBytes / 1024;  // 1-KiB direct-to-LDS loads per stage
+    static constexpr int CH = CHUNKS / NWAVES;         // per wave
+    static constexpr int STORES = FM * FN * 16;        // dword stores per lane per tile
+    static constexpr int SLOTS = FM * FN;              // MFMAs per unit (one k-fragment)
+    static_assert(CHUNKS % NWAVES == 0 && CH % 2 == 0 && CH <= 63, "loads must split evenly");
+};
+
+template <class C>
+__global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
+    const uint8_t *__restrict__ XW, const uint8_t *__restrict__ WW, int32_t *__restrict__ Y,
+    int M, int N, int K, int tiles_m, int tiles_n)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wm = wave / C::WAVES_N;
+    const int wn = wave % C::WAVES_N;
+    const int KT = K / kStageK;
+    const int total_tiles = tiles_m * tiles_n;
+    const int nblk = gridDim.x;
+    const int bid = blockIdx.x;
+    if (bid >= total_tiles)
+        return;
+    const int my_tiles = (total_tiles - bid + nblk - 1) / nblk;
+    const int total_stages = my_tiles * KT;
+
+    // ---- load side: stage = 24 KiB of X fragments then 24 KiB of W fragments, copied
+    //      linearly; wave w moves the 1-KiB chunks w, w + NWAVES, ...
+    const uint8_t *xptr = XW, *wptr = WW;  // wave-uniform: this tile's current stage
+    int ld_it = 0, ld_k = 0, issued = 0;
+    const unsigned lds_base = (unsigned)(size_t)I4L_LDS(lds);
+    const unsigned lane16 = (unsigned)lane * 16u;
+
+    auto ld_setup_tile = [&](int it) {
+        int tm, tn;
+        tile_coords(bid + it * nblk, total_tiles, tiles_m, tiles_n, tm, tn);
+        xptr = XW + (size_t)tm * KT * kOperandStageBytes;
+        wptr = WW + (size_t)tn * KT * kOperandStageBytes;
+    };
+    auto ld_chunk = [&](int c) {
+        const int q = c * C::NWAVES + wave;  // chunk of the stage, 0 .. CHUNKS-1
+        const bool is_x = q < C::CHUNKS / 2;
+        const uint8_t *src = is_x ? xptr + q * 1024 : wptr + (q - C::CHUNKS / 2) * 1024;
+        dma16(src, lane16, lds_base + (issued % kStages) * kStageBytes + q * 1024);
+    };
+    auto ld_advance = [&]() {
+        ++issued;
+        ++ld_k;
+        xptr += kOperandStageBytes;
+        wptr += kOperandStageBytes;
+        if (ld_k == KT) {
+            ld_k = 0;
+            ++ld_it;
+            if (ld_it < my_tiles)
+                ld_setup_tile(ld_it);
+        }
+    };
+
+    ld_setup_tile(0);
+#pragma unroll 1
+    for (int s = 0; s < kStages; ++s)
+        if (issued < total_stages) {
+#pragma unroll
+            for (int c = 0; c < C::CH; ++c)
+                ld_chunk(c);
+            ld_advance();
+        }
+
+    // ---- math side.  Unit u = (stage, k-fragment kf); its operands are FM X fragments
+    //      and FN W fragments, each 6 VGPRs read as 16 + 8 bytes.  While the MFMAs of unit
+    //      u run, the fragments of unit u+1 are read into the other register set.
+    const unsigned x_rd = (unsigned)(wm * C::FM * kFragBytes) + lane16;
+    const unsigned w_rd = (unsigned)(kOperandStageBytes + wn * C::FN * kFragBytes) + lane16;
+    const unsigned hi_delta = (unsigned)kFragLoBytes - (unsigned)lane * 8u;  // from the 16-B to the 8-B part
+
+    v16f acc[C::FN][C::FM];
+    v4i xlo[2][C::FM], wlo[2][C::FN];  // first 128 bits of each fragment's 192
+    v2i xhi[2][C::FM], whi[2][C::FN];  // last 64 bits
+    int cur_it = 0, kk = 0;
+
+    // Read instruction r (0 .. 2*(FM+FN)-1) of unit (st, kf) into register set p:
+    // fragment r/2, 16-byte part for even r, 8-byte part for odd r; X fragments first.
+    auto read_op = [&](int st, int kf, int p, int r) {
+        const uint8_t *base = lds + (st % kStages) * kStageBytes + kf * kFragsRows * kFragBytes;
+        const int f = r >> 1;
+        const bool is_x = f < C::FM;
+        const int idx = is_x ? f : f - C::FM;
+        const uint8_t *a = base + (is_x ? x_rd : w_rd) + idx * kFragBytes;
+        if ((r & 1) == 0)
+            (is_x ? xlo[p][idx] : wlo[p][idx]) = *(const v4i *)a;
+        else
+            (is_x ? xhi[p][idx] : whi[p][idx]) = *(const v2i *)(a + hi_delta);
+    };
+    auto frag = [](const v4i &lo, const v2i &hi) {
+        return (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], 0, 0};
+    };
+    constexpr int kReads = 2 * (C::FM + C::FN);
+
+    // The MFMAs of the unit held in register set p; `hook(slot)` is housekeeping placed
+    // behind the MFMA of that slot.
+    auto unit = [&](auto p_tag, auto &&hook) {
+        constexpr int p = decltype(p_tag)::value;
+        [&]<int... SLOT>(std::integer_sequence<int, SLOT...>) {
+            ([&] {
+                constexpr int j = SLOT / C::FN, i = SLOT % C::FN;
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                    frag(xlo[p][j], xhi[p][j]), frag(wlo[p][i], whi[p][i]), acc[i][j], 2, 2, 0, kScale, 0,
+                    kScale);
+                __builtin_amdgcn_sched_barrier(0);
+                hook(std::integral_constant<int, SLOT>{});
+                __builtin_amdgcn_sched_barrier(0);
+            }(), ...);
+        }(std::make_integer_sequence<int, C::SLOTS>{});
+    };
+
+    // Housekeeping positions inside a unit of SLOTS slots: the kReads LDS reads of the
+    // next unit go two per slot from slot 0 (so they have landed well before the unit
+    // ends), the CH/2 direct-to-LDS loads one per slot from slot SLOTS/2.
+    constexpr int kReadsPerSlot = 2;
+    constexpr int kDmaFirstSlot = C::SLOTS / 2;
+    static_assert(kReads <= kReadsPerSlot * C::SLOTS, "not enough slots for the LDS reads");
+    static_assert(kDmaFirstSlot + C::CH / 2 <= C::SLOTS, "not enough slots for the loads");
+    bool loading = false;
+    auto spread = [&](auto slot_tag, int read_st, int read_kf, int read_p, int half_pos) {
+        constexpr int slot = decltype(slot_tag)::value;
+#pragma unroll
+        for (int r = slot * kReadsPerSlot; r < (slot + 1) * kReadsPerSlot && r < kReads; ++r)
+            read_op(read_st, read_kf, read_p, r);
+        if constexpr (slot >= kDmaFirstSlot && slot < kDmaFirstSlot + C::CH / 2) {
+            if (loading)
+                ld_chunk(half_pos * (C::CH / 2) + slot - kDmaFirstSlot);
+        }
+    };
+
+    // Stage 0 must have landed before the first read.
+    if (issued >= kStages)
+        __builtin_amdgcn_s_waitcnt(I4L_WAIT_VM((kStages - 1) * C::CH));
+    else
+        __builtin_amdgcn_s_waitcnt(I4L_WAIT_VM(0));
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int r = 0; r < kReads; ++r)
+        read_op(0, 0, 0, r);
+
+#pragma unroll 1
+    for (int gs = 0; gs < total_stages; ++gs) {
+        if (kk == 0) {
+#pragma unroll
+            for (int i = 0; i < C::FN; ++i)
+#pragma unroll
+                for (int j = 0; j < C::FM; ++j)
+#pragma unroll
+                    for (int t = 0; t < 16; ++t)
+                        acc[i][j][t] = 0.f;
+        }
+
+        // ---- unit (gs, 0): reads unit (gs, 1); finishes the loads begun last iteration
+        unit(std::integral_constant<int, 0>{}, [&](auto slot_tag) {
+            spread(slot_tag, gs, 1, 1, 1);
+            if constexpr (decltype(slot_tag)::value == C::SLOTS - 1) {
+                if (loading) {
+                    ld_advance();
+                    loading = false;
+                }
+            }
+        });
+
+        // ---- between the units: every LDS read of stage gs has been issued; once they
+        //      have returned (lgkmcnt 0) and every wave is here, the buffer of stage gs is
+        //      free for stage gs+3.  Stage gs+1 must have landed: loads complete in order,
+        //      normally one younger stage (gs+2) is in flight behind it, and in the first
+        //      stage after a tile end that tile's C stores sit behind it as well.
+        {
+            const int ahead = issued - 2 - gs;  // stages issued after stage gs+1
+            if (ahead >= 1) {
+                if (cur_it > 0 && kk < 1) {
+                    constexpr int with_stores = C::CH + C::STORES;
+                    __builtin_amdgcn_s_waitcnt(I4L_WAIT_VM_LGKM0(with_stores < 63 ? with_stores : 63));
+                } else {
+                    __builtin_amdgcn_s_waitcnt(I4L_WAIT_VM_LGKM0(C::CH));
+                }
+            } else {
+                __builtin_amdgcn_s_waitcnt(I4L_WAIT_VM_LGKM0(0));
+            }
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            loading = issued < total_stages;
+        }
+
+        // ---- unit (gs, 1): reads unit (gs+1, 0) (a stale buffer past the last stage, never
+        //      multiplied into a stored tile); begins the loads of stage gs+3
+        unit(std::integral_constant<int, 1>{}, [&](auto slot_tag) { spread(slot_tag, gs + 1, 0, 0, 0); });
+
+        ++kk;
+        if (kk == KT) {
+            // ---- store the tile.  X is the MFMA A operand: accumulator t of tile (i, j) is
+            //   m = 32*j + 8*(t/4) + 4*(lane/32) + t%4,  n = 32*i + lane%32,
+            // so one dword store writes two rows of 32 consecutive n (128 B each).
+            int tm, tn;
+            tile_coords(bid + cur_it * nblk, total_tiles, tiles_m, tiles_n, tm, tn);
+            const int m0 = tm * kTileRows, n0 = tn * kTileRows;
+            const int rows_left = M - m0;  // > 0
+            const int cols_left = N - n0;  // > 0
+            int32_t *ybase = Y + (size_t)m0 * N + n0;
+            const size_t slab_rows = rows_left < kTileRows ? rows_left : kTileRows;
+            const size_t extent = ((slab_rows - 1) * (size_t)N + (size_t)(cols_left < kTileRows ? cols_left : kTileRows)) * 4u;
+            __amdgpu_buffer_rsrc_t rsrc =
+                __builtin_amdgcn_make_buffer_rsrc(ybase, 0, (int)extent, 0x00020000);
+            // A lane outside the matrix gets an offset part so large that the sum falls
+            // outside the descriptor's range and the hardware drops the store.
+            const int lm = opaque(wm * C::FM * kFragRows + (lane >> 5) * 4);
+            const int ln = opaque(wn * C::FN * kFragRows + (lane & 31));
+            const unsigned lm_off = (unsigned)lm * (unsigned)N * 4u;
+            unsigned col_off[C::FN];
+#pragma unroll
+            for (int i = 0; i < C::FN; ++i) {
+                const int ncol = ln + i * kFragRows;
+                col_off[i] = ncol < cols_left ? (unsigned)ncol * 4u : 0x40000000u;
+            }
+#pragma unroll
+            for (int j = 0; j < C::FM; ++j) {
+#pragma unroll
+                for (int t = 0; t < 16; ++t) {
+                    const int dm = j * kFragRows + 8 * (t / 4) + (t % 4);  // uniform
+                    const unsigned row_off = lm + dm < rows_left ? lm_off + (unsigned)dm * (unsigned)N * 4u : 0x80000000u;
+#pragma unroll
+                    for (int i = 0; i < C::FN; ++i) {
+                        const int v = (int)acc[i][j][t];  // exact: the accumulator holds an integer
+                        __builtin_amdgcn_raw_buffer_store_b32((unsigned)v, rsrc, row_off + col_off[i], 0, 2 /* nt */);
+                    }
+                }
+            }
+            kk = 0;
+            ++cur_it;
+        }
+    }
+}
+
+// Eight wavefronts of 128 (m) x 64 (n), two per SIMD, one workgroup per CU.
+using Fp6Cfg = Fp6Config<2, 4, 1>;
+
+size_t operand_ws_bytes(int rows, int k)
+{
+    const size_t tiles = (size_t)(rows + kTileRows - 1) / kTileRows;
+    return tiles * (size_t)(k / kStageK) * (size_t)kOperandStageBytes;
+}
+
+}  // namespace
+
+bool fp6_supports(int m, int n, int k)
+{
+    // fp32 accumulation of products bounded by 64 stays exact while K * 64 < 2^24.
+    return m >= 1 && n >= 1 && k >= kStageK && k % kStageK == 0 && k < (1 << 18);
+}
+
+size_t fp6_workspace_bytes(int m, int n, int k)
+{
+    return operand_ws_bytes(m, k) + operand_ws_bytes(n, k);
+}
+
+hipError_t fp6_init(const DeviceInfo &dev)
+{
+    if (dev.lds_per_cu < kLdsBytes)
+        return hipErrorInvalidConfiguration;
+    return hipFuncSetAttribute((const void *)fp6_gemm_kernel<Fp6Cfg>,
+                               hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+}
+
+hipError_t launch_fp6(const void *a, const void *b, void *c, int m, int n, int k, void *workspace,
+                      const DeviceInfo &dev, hipStream_t stream)
+{
+    using C = Fp6Cfg;
+    uint8_t *xws = (uint8_t *)workspace;
+    uint8_t *wws = xws + operand_ws_bytes(m, k);
+    const int tiles_m = (m + kTileRows - 1) / kTileRows;
+    const int tiles_n = (n + kTileRows - 1) / kTileRows;
+    const long total = (long)tiles_m * tiles_n;
+    if (total > 0x7fffffffL || (size_t)kTileRows * (size_t)n * 4u > 0x40000000ull)
+        return hipErrorInvalidValue;
+    if (tiles_m * 8 > 65535 || tiles_n * 8 > 65535)
+        return hipErrorInvalidValue;
+
+    // One converter workgroup per 32 rows x 256 k (K % 256 may be 128: the kernel guards).
+    const int kblocks = (k + 255) / 256;
+    fp6_convert_kernel<<<dim3(kblocks, tiles_m * kFragsRows), 256, 0, stream>>>(
+        (const uint8_t *)a, xws, m, tiles_m * kTileRows, k);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess)
+        return e;
+    fp6_convert_kernel<<<dim3(kblocks, tiles_n * kFragsRows), 256, 0, stream>>>(
+        (const uint8_t *)b, wws, n, tiles_n * kTileRows, k);
+    e = hipGetLastError();
+    if (e != hipSuccess)
+        return e;
+
+    long grid = (long)dev.cu_count * C::OCC;
+    if (grid > total)
+        grid = total;
+    fp6_gemm_kernel<C><<<(unsigned)grid, C::THREADS, kLdsBytes, stream>>>(
+        xws, wws, (int32_t *)c, m, n, k, tiles_m, tiles_n);
+    return hipGetLastError();
+}
+
+}  // namespace int4linear

@@ -17,6 +17,7 @@ def kernels_for(m, n, k):
     ks = ["auto", "simple"]
     if k >= 128 and k % 128 == 0:
         ks.append("mfma")
+        ks.append("fp6")
         if m <= 64:
             ks.append("skinny")
     return ks
@@ -72,6 +73,11 @@ def test_cfg2_cfg3_large(gpu, host_threads, m, n, k):
     # the whole matrix against the independent scalar kernel, on the device
     ref_d = helpers.run_gemm(xp, wp, m, n, k, kernel="simple", keep_on_device=True)
     assert torch.equal(got_d, ref_d)
+    del got_d
+    for kern in ("mfma", "fp6"):
+        other = helpers.run_gemm(xp, wp, m, n, k, kernel=kern, keep_on_device=True)
+        assert torch.equal(other, ref_d), kern
+        del other
 
 
 # ---- configuration 4: decode shapes ------------------------------------------------------
@@ -83,7 +89,7 @@ def test_cfg4_decode(gpu, host_threads, m, n, k):
     w = helpers.uniform_s4(400 + n + k, n, k)      # weights: uniform [-8, 7]
     want = oracle.linear_ref(x, w, threads=host_threads)
     xp, wp = helpers.pack_bytes(x), helpers.pack_bytes(w)
-    for kern in ("auto", "skinny", "mfma"):
+    for kern in ("auto", "skinny", "mfma", "fp6"):
         got = helpers.run_gemm(xp, wp, m, n, k, kernel=kern)
         assert np.array_equal(got, want), f"kernel={kern}"
 
@@ -96,17 +102,17 @@ def test_cfg5_all_minus_eight_full_size(gpu):
     m, n, k = 8192, 28672, 8192
     xp = np.full((m, k // 2), 0x88, dtype=np.uint8)
     wp = np.full((n, k // 2), 0x88, dtype=np.uint8)
-    got = helpers.run_gemm(xp, wp, m, n, k, kernel="auto", keep_on_device=True)
-    assert bool((got == 524288).all())
-    assert int(got.min()) == 524288 and int(got.max()) == 524288
-    del got
-    torch.cuda.empty_cache()
+    for kern in ("auto", "mfma", "fp6"):
+        got = helpers.run_gemm(xp, wp, m, n, k, kernel=kern, keep_on_device=True)
+        assert int(got.min()) == 524288 and int(got.max()) == 524288, kern
+        del got
+        torch.cuda.empty_cache()
 
 
 def test_cfg5_ragged_1000_3000_4096(gpu, host_threads):
     x = helpers.uniform_s4(51, 1000, 4096)
     w = helpers.uniform_s4(52, 3000, 4096)
-    check_all_kernels(x, w, threads=host_threads, kernels=["auto", "mfma", "simple"])
+    check_all_kernels(x, w, threads=host_threads, kernels=["auto", "mfma", "fp6", "simple"])
 
 
 @pytest.mark.parametrize("a, b, per_k", [(-8, -8, 64), (7, 7, 49), (-8, 7, -56), (7, -8, -56)])

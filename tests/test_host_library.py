@@ -72,10 +72,13 @@ def test_null_and_alignment_checks():
     assert L.int4linear_gemm_s4s4s32(16, 16, 24, 4, 4, 8, None) == 3            # C misaligned
     assert L.int4linear_gemm_s4s4s32(8, 16, 16, 4, 4, 8, None) == 3             # A misaligned
     assert L.int4linear_gemm_s4s4s32_ex(16, 16, 16, 4, 4, 8, 9, None) == 5      # unknown kernel
+    assert L.int4linear_gemm_s4s4s32_ex(16, 16, 16, 4, 4, 8, -1, None) == 5
 
 
 def test_kernel_dispatch_table():
-    assert lib.kernel_for_shape(8192, 8192, 8192) == "mfma"
+    assert lib.kernel_for_shape(8192, 8192, 8192) == "fp6"
+    assert lib.kernel_for_shape(4096, 4096, 4096) == "fp6"
+    assert lib.kernel_for_shape(2048, 2048, 2048) == "mfma"   # too few 256 x 256 tiles
     assert lib.kernel_for_shape(1024, 1024, 1024) == "mfma"
     assert lib.kernel_for_shape(1000, 3000, 4096) == "mfma"
     assert lib.kernel_for_shape(16, 4096, 4096) == "skinny"
@@ -85,6 +88,21 @@ def test_kernel_dispatch_table():
     assert lib.kernel_for_shape(128, 128, 64) == "simple"     # K below one pipeline stage
     assert lib.kernel_for_shape(128, 128, 200) == "simple"    # K % 128 != 0
     assert lib.kernel_for_shape(4, 4, 12) == "invalid"
+
+
+def test_workspace_accounting():
+    # FP6 workspace: both operands, rows padded to 256, 0.75 byte per element
+    assert lib.workspace_bytes(8192, 8192, 8192) == 2 * 8192 * 8192 * 3 // 4
+    assert lib.workspace_bytes(4000, 8192, 4096) == (4096 + 8192) * 4096 * 3 // 4
+    assert lib.workspace_bytes(16, 4096, 4096) == 0      # skinny kernel: none
+    assert lib.workspace_bytes(1024, 1024, 1024) == 0    # int8 kernel: none
+    lib.set_workspace_limit(0)
+    try:
+        assert lib.workspace_bytes(8192, 8192, 8192) == 0
+        assert lib.kernel_for_shape(8192, 8192, 8192) == "mfma"
+    finally:
+        lib.set_workspace_limit(1 << 30)
+    assert lib.kernel_for_shape(8192, 8192, 8192) == "fp6"
 
 
 @pytest.mark.parametrize("m, n, seed", [(1, 8, 1), (3, 10, 2), (16, 64, 3), (7, 129, 4), (64, 4096, 5)])
