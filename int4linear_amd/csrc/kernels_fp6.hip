@@ -222,22 +222,34 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
         xptr += kOperandStageBytes;
         wptr += kOperandStageBytes;
         if (ld_k == KT) {
-            ld_k = 0;
-            ++ld_it;
-            if (ld_it < my_tiles)
+            if (ld_it + 1 < my_tiles) {
+                ld_k = 0;
+                ++ld_it;
                 ld_setup_tile(ld_it);
+            } else {
+                // Past the last stage the cursor stays on it: the loop keeps issuing loads
+                // unconditionally, and these re-read valid data into buffers nobody reads.
+                ld_k = KT - 1;
+                xptr -= kOperandStageBytes;
+                wptr -= kOperandStageBytes;
+            }
         }
     };
 
+    // Prologue: stages 0 and 1 in full and the first half of stage 2's loads.  From then on
+    // every iteration gs finishes stage gs+2 in its first unit and begins stage gs+3 in its
+    // second, so the loop body needs no branch around a load.
     ld_setup_tile(0);
-#pragma unroll 1
-    for (int s = 0; s < kStages; ++s)
-        if (issued < total_stages) {
 #pragma unroll
-            for (int c = 0; c < C::CH; ++c)
-                ld_chunk(c);
-            ld_advance();
-        }
+    for (int s = 0; s < kStages - 1; ++s) {
+#pragma unroll
+        for (int c = 0; c < C::CH; ++c)
+            ld_chunk(c);
+        ld_advance();
+    }
+#pragma unroll
+    for (int c = 0; c < C::CH / 2; ++c)
+        ld_chunk(c);
 
     // ---- math side.  Unit u = (stage, k-fragment kf); its operands are FM X fragments
     //      and FN W fragments, each 6 VGPRs read as 16 + 8 bytes.  While the MFMAs of unit
@@ -293,23 +305,19 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
     constexpr int kDmaFirstSlot = C::SLOTS / 2;
     static_assert(kReads <= kReadsPerSlot * C::SLOTS, "not enough slots for the LDS reads");
     static_assert(kDmaFirstSlot + C::CH / 2 <= C::SLOTS, "not enough slots for the loads");
-    bool loading = false;
     auto spread = [&](auto slot_tag, int read_st, int read_kf, int read_p, int half_pos) {
         constexpr int slot = decltype(slot_tag)::value;
 #pragma unroll
         for (int r = slot * kReadsPerSlot; r < (slot + 1) * kReadsPerSlot && r < kReads; ++r)
             read_op(read_st, read_kf, read_p, r);
         if constexpr (slot >= kDmaFirstSlot && slot < kDmaFirstSlot + C::CH / 2) {
-            if (loading)
-                ld_chunk(half_pos * (C::CH / 2) + slot - kDmaFirstSlot);
+            ld_chunk(half_pos * (C::CH / 2) + slot - kDmaFirstSlot);
         }
     };
 
-    // Stage 0 must have landed before the first read.
-    if (issued >= kStages)
-        __builtin_amdgcn_s_waitcnt(I4L_WAIT_VM((kStages - 1) * C::CH));
-    else
-        __builtin_amdgcn_s_waitcnt(I4L_WAIT_VM(0));
+    // Stage 0 must have landed before the first read; stage 1 and half of stage 2 are
+    // in flight behind it.
+    __builtin_amdgcn_s_waitcnt(I4L_WAIT_VM(C::CH + C::CH / 2));
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 #pragma unroll
@@ -328,15 +336,11 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
                         acc[i][j][t] = 0.f;
         }
 
-        // ---- unit (gs, 0): reads unit (gs, 1); finishes the loads begun last iteration
+        // ---- unit (gs, 0): reads unit (gs, 1); finishes the loads of stage gs+2
         unit(std::integral_constant<int, 0>{}, [&](auto slot_tag) {
             spread(slot_tag, gs, 1, 1, 1);
-            if constexpr (decltype(slot_tag)::value == C::SLOTS - 1) {
-                if (loading) {
-                    ld_advance();
-                    loading = false;
-                }
-            }
+            if constexpr (decltype(slot_tag)::value == C::SLOTS - 1)
+                ld_advance();
         });
 
         // ---- between the units: every LDS read of stage gs has been issued; once they
@@ -345,24 +349,19 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
         //      normally one younger stage (gs+2) is in flight behind it, and in the first
         //      stage after a tile end that tile's C stores sit behind it as well.
         {
-            const int ahead = issued - 2 - gs;  // stages issued after stage gs+1
-            if (ahead >= 1) {
-                if (cur_it > 0 && kk < 1) {
-                    constexpr int with_stores = C::CH + C::STORES;
-                    __builtin_amdgcn_s_waitcnt(I4L_WAIT_VM_LGKM0(with_stores < 63 ? with_stores : 63));
-                } else {
-                    __builtin_amdgcn_s_waitcnt(I4L_WAIT_VM_LGKM0(C::CH));
-                }
+            if (cur_it > 0 && kk < 1) {
+                constexpr int with_stores = C::CH + C::STORES;
+                __builtin_amdgcn_s_waitcnt(I4L_WAIT_VM_LGKM0(with_stores < 63 ? with_stores : 63));
             } else {
-                __builtin_amdgcn_s_waitcnt(I4L_WAIT_VM_LGKM0(0));
+                __builtin_amdgcn_s_waitcnt(I4L_WAIT_VM_LGKM0(C::CH));
             }
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
-            loading = issued < total_stages;
         }
 
         // ---- unit (gs, 1): reads unit (gs+1, 0) (a stale buffer past the last stage, never
-        //      multiplied into a stored tile); begins the loads of stage gs+3
+        //      multiplied into a stored tile); begins the loads of stage gs+3 into the
+        //      buffer of stage gs
         unit(std::integral_constant<int, 1>{}, [&](auto slot_tag) { spread(slot_tag, gs + 1, 0, 0, 0); });
 
         ++kk;
