@@ -51,6 +51,19 @@ def _run(cmd: list[str]) -> None:
         sys.stderr.write(out + "\n")
 
 
+def _check_no_missing_kernels() -> None:
+    """A kernel whose device or host half failed to be emitted shows up as an undefined
+    symbol of this project's namespace; refuse such a library."""
+    nm = shutil.which("nm")
+    if not nm:
+        return
+    out = subprocess.run([nm, "-D", "--undefined-only", str(LIB_PATH)], stdout=subprocess.PIPE,
+                         text=True).stdout
+    missing = [l.split()[-1] for l in out.splitlines() if "int4linear" in l]
+    if missing:
+        raise RuntimeError("libint4linear.so has undefined project symbols: " + ", ".join(missing))
+
+
 def build_library(verbose: bool = False, save_temps: bool = False) -> Path:
     """Compile every source and link the shared library.  Always recompiles."""
     hipcc = _hipcc()
@@ -76,6 +89,7 @@ def build_library(verbose: bool = False, save_temps: bool = False) -> Path:
     if verbose:
         print(" ".join(link))
     _run(link)
+    _check_no_missing_kernels()
     return LIB_PATH
 
 

@@ -137,6 +137,9 @@ __device__ __forceinline__ void dma16(const void *sbase, unsigned voff, unsigned
                  : "memory");
 }
 
+// Marks a value as used at this point of the program without generating code.
+__device__ __forceinline__ void pin(const v16f &v) { asm volatile("" ::"v"(v)); }
+
 __device__ __forceinline__ int opaque(int v)
 {
     asm volatile("" : "+v"(v));
@@ -258,6 +261,14 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
     const unsigned w_rd = (unsigned)(kOperandStageBytes + wn * C::FN * kFragBytes) + lane16;
     const unsigned hi_delta = (unsigned)kFragLoBytes - (unsigned)lane * 8u;  // from the 16-B to the 8-B part
 
+#ifdef I4L_EXP_TRACE
+    long long *trace = (long long *)(lds + kLdsBytes);
+    int trace_n = 0;
+    const bool tracer = (bid == 0) && (threadIdx.x == I4L_EXP_TRACE * 64);
+#define I4L_STAMP() do { if (tracer && trace_n < 1900) { trace[trace_n++] = __builtin_readcyclecounter(); } } while (0)
+#else
+#define I4L_STAMP() do {} while (0)
+#endif
     v16f acc[C::FN][C::FM];
     v4i xlo[2][C::FM], wlo[2][C::FN];  // first 128 bits of each fragment's 192
     v2i xhi[2][C::FM], whi[2][C::FN];  // last 64 bits
@@ -291,6 +302,10 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
                 acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
                     frag(xlo[p][j], xhi[p][j]), frag(wlo[p][i], whi[p][i]), acc[i][j], 2, 2, 0, kScale, 0,
                     kScale);
+                // An MFMA has no side effect, so nothing stops the optimiser from moving it
+                // down to its next use, past the housekeeping meant to run in its shadow;
+                // this empty statement "uses" the result here and keeps the MFMA in place.
+                pin(acc[i][j]);
                 __builtin_amdgcn_sched_barrier(0);
                 hook(std::integral_constant<int, SLOT>{});
                 __builtin_amdgcn_sched_barrier(0);
@@ -326,6 +341,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
 
 #pragma unroll 1
     for (int gs = 0; gs < total_stages; ++gs) {
+        I4L_STAMP();
         if (kk == 0) {
 #pragma unroll
             for (int i = 0; i < C::FN; ++i)
@@ -349,13 +365,16 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
         //      normally one younger stage (gs+2) is in flight behind it, and in the first
         //      stage after a tile end that tile's C stores sit behind it as well.
         {
+            I4L_STAMP();
             if (cur_it > 0 && kk < 1) {
                 constexpr int with_stores = C::CH + C::STORES;
                 __builtin_amdgcn_s_waitcnt(I4L_WAIT_VM_LGKM0(with_stores < 63 ? with_stores : 63));
             } else {
                 __builtin_amdgcn_s_waitcnt(I4L_WAIT_VM_LGKM0(C::CH));
             }
+            I4L_STAMP();
             __builtin_amdgcn_s_barrier();
+            I4L_STAMP();
             asm volatile("" ::: "memory");
         }
 
@@ -364,6 +383,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
         //      buffer of stage gs
         unit(std::integral_constant<int, 1>{}, [&](auto slot_tag) { spread(slot_tag, gs + 1, 0, 0, 0); });
 
+        I4L_STAMP();
         ++kk;
         if (kk == KT) {
             // ---- store the tile.  X is the MFMA A operand: accumulator t of tile (i, j) is
@@ -407,6 +427,16 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
             ++cur_it;
         }
     }
+#ifdef I4L_EXP_TRACE
+    I4L_STAMP();
+    __builtin_amdgcn_s_waitcnt(0);
+    if (tracer) {
+        long long *dst = (long long *)Y;
+        dst[0] = trace_n;
+        for (int i = 0; i < trace_n; ++i)
+            dst[1 + i] = trace[i];
+    }
+#endif
 }
 
 // Eight wavefronts of 128 (m) x 64 (n), two per SIMD, one workgroup per CU.
@@ -469,6 +499,12 @@ hipError_t launch_fp6(const void *a, const void *b, void *c, int m, int n, int k
     long grid = (long)dev.cu_count * C::OCC;
     if (grid > total)
         grid = total;
+#ifdef I4L_EXP_TRACE
+    hipFuncSetAttribute((const void *)fp6_gemm_kernel<C>, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes + 16000);
+    fp6_gemm_kernel<C><<<(unsigned)grid, C::THREADS, kLdsBytes + 16000, stream>>>(
+        xws, wws, (int32_t *)c, m, n, k, tiles_m, tiles_n);
+    return hipGetLastError();
+#endif
     fp6_gemm_kernel<C><<<(unsigned)grid, C::THREADS, kLdsBytes, stream>>>(
         xws, wws, (int32_t *)c, m, n, k, tiles_m, tiles_n);
     return hipGetLastError();
