@@ -65,6 +65,8 @@ int ensure_init(PerDevice **out)
         err = mfma_init(pd.info);
         if (err == hipSuccess)
             err = fp6_init(pd.info);
+        if (err == hipSuccess)
+            err = skinny_init(pd.info);
         if (err != hipSuccess) {
             pd.init_error = err;
             pd.status = INT4LINEAR_ERR_HIP;

@@ -31,6 +31,7 @@ hipError_t launch_fp6(const void *a, const void *b, void *c, int m, int n, int k
 
 // Weight-streaming kernel for skinny M.  Requires M <= 64, K % 128 == 0.
 bool skinny_supports(int m, int n, int k);
+hipError_t skinny_init(const DeviceInfo &dev);
 hipError_t launch_skinny(const void *a, const void *b, void *c, int m, int n, int k,
                          const DeviceInfo &dev, hipStream_t stream);
 

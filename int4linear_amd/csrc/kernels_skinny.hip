@@ -1,15 +1,24 @@
-// Weight-streaming kernel for skinny M (M <= 64): the decode-shaped linear layer.
+// Weight-streaming kernels for skinny M (M <= 64): the decode-shaped linear layer.
 //
-// The job is HBM-bound: every byte of W (N x K/2) is read exactly once, straight from
-// global memory into registers with 16-byte loads, widened to int8 (same 16x trick as
-// the big kernel: (w << 4) & 0xF0F0F0F0 and w & 0xF0F0F0F0) and multiplied on
-// v_mfma_i32_16x16x64_i8 against X, which is small enough to live in L2.
+// The job is HBM-bound: every byte of W (N x K/2) is read exactly once and the arithmetic
+// (v_mfma_i32_16x16x64_i8 after the same 16x nibble widening as the big int8 kernel:
+// (w << 4) & 0xF0F0F0F0 and w & 0xF0F0F0F0, C = acc >> 8) is free next to it.  What decides
+// the speed is the shape of the global reads.  Measured on MI355X for a 28 MiB weight
+// matrix: a wave instruction whose eight-lane groups each read one whole 128-byte line
+// streams as fast as a plain linear read, while the natural MFMA pattern (sixteen rows,
+// 64 bytes of each) is 25 % slower.  So W is not loaded in MFMA layout.  Each load
+// instruction moves eight rows x 128 bytes straight into LDS (global_load_lds_dwordx4,
+// non-temporal), and the MFMA operands are read back from LDS in fragment layout; a
+// 16-byte XOR swizzle of the slot index (applied by permuting which global chunk a lane
+// fetches, since the LDS position of a lane's data is fixed) keeps those reads free of
+// bank conflicts.
 //
-// A workgroup owns 16 consecutive rows of W (16 columns of C) -- one contiguous
-// 16 * K/2-byte slab -- and its wavefronts split K between them, interleaved by
-// 128-nibble steps so each round of the workgroup reads 64*WAVES contiguous bytes of
-// every row.  Partial sums meet in LDS; one pass adds them and stores C.  No atomics,
-// no workspace, and the result does not depend on timing.
+// A workgroup owns R groups of 16 consecutive rows of W (16*R columns of C) over the
+// whole of K.  Its S wavefronts split K into S slices of T tiles of 256 nibbles; a wave
+// issues every load of its slices before it waits for anything, multiplies, and the S
+// partial sums meet once in LDS.  Each wave fetches its own slice of X once and reuses it
+// for its R row groups, so larger R cuts the (L2-resident, but hot-line) X traffic.
+// No atomics, no workspace, and the result does not depend on timing.
 #include "kernels.h"
 
 namespace int4linear {
@@ -18,25 +27,189 @@ namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 
-constexpr int kStepK = 128;         // nibbles per wave step
-constexpr int kStepBytes = 64;      // bytes per row per step
-constexpr int kBatch = 4;           // steps whose loads are issued together
+#define I4L_LDS(p) ((__attribute__((address_space(3))) void *)(p))
 
+constexpr int kTileK = 256;                 // nibbles of K per tile
+constexpr int kTileRowBytes = kTileK / 2;   // one 128-byte line per row
+constexpr int kTileBytes = 16 * kTileRowBytes;  // 16 rows: 2 KiB
+constexpr int kMaxLds = 160 * 1024;
+
+// 16 bytes per lane from a per-lane global address straight into LDS at lds_addr +
+// 16*lane.  NT marks the weight stream as read-once.
+template <bool NT>
+__device__ __forceinline__ void dma16(const void *gptr, unsigned lds_addr)
+{
+    if (NT)
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt"
+                     :
+                     : "v"(gptr), "s"(lds_addr)
+                     : "memory");
+    else
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                     :
+                     : "v"(gptr), "s"(lds_addr)
+                     : "memory");
+}
+
+// LDS slot (16 bytes) of chunk c of tile row r: c ^ ((r >> 1) & 7).  Rows are 128 B apart,
+// so the sixteen lanes that read one chunk of rows 0..15 hit sixteen different 16-byte
+// bank groups of the 256-byte bank window.
+__device__ __forceinline__ int slot_swizzle(int r) { return (r >> 1) & 7; }
+
+// T tiles per wave, R row groups per workgroup, FMX 16-row groups of X (M <= 16*FMX).
+// XDMA: X tiles go through LDS like W; otherwise they are loaded into registers in
+// fragment layout (for K so long that X tiles do not fit in LDS next to the W staging).
+template <int T, int R, int FMX, bool XDMA>
+__global__ __launch_bounds__(1024) void skinny_kernel(const uint8_t *__restrict__ X,
+                                                      const uint8_t *__restrict__ W,
+                                                      int32_t *__restrict__ Y, int M, int N, int K)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    constexpr int kWaveTiles = T * (R + (XDMA ? FMX : 0));
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int waves = blockDim.x >> 6;  // S
+    const int rowbytes = K >> 1;
+    const int n0 = blockIdx.x * 16 * R;
+    const unsigned lds_base = (unsigned)(size_t)I4L_LDS(lds);
+    const unsigned my_lds = lds_base + wave * kWaveTiles * kTileBytes;
+    const size_t kbyte0 = (size_t)wave * T * kTileRowBytes;  // this wave's slice of every row
+
+    // ---- loads.  Lane p of a load instruction lands in LDS at 16*p: tile row p/8 (+8 for
+    //      the second instruction of a tile), slot p%8, so it fetches chunk slot ^ swizzle.
+    {
+        const int lrow = lane >> 3;
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int row = lrow + 8 * u;
+            const int chunk = (lane & 7) ^ slot_swizzle(row);
+#pragma unroll
+            for (int rg = 0; rg < R; ++rg) {
+                const int wr = n0 + rg * 16 + row;
+                const uint8_t *src = W + (size_t)(wr < N ? wr : N - 1) * rowbytes + kbyte0 + chunk * 16;
+#pragma unroll
+                for (int t = 0; t < T; ++t)
+                    dma16<true>(src + t * kTileRowBytes, my_lds + (rg * T + t) * kTileBytes + u * 1024);
+            }
+            if (XDMA) {
+#pragma unroll
+                for (int f = 0; f < FMX; ++f) {
+                    const int xr = f * 16 + row;
+                    const uint8_t *src = X + (size_t)(xr < M ? xr : M - 1) * rowbytes + kbyte0 + chunk * 16;
+#pragma unroll
+                    for (int t = 0; t < T; ++t)
+                        dma16<false>(src + t * kTileRowBytes,
+                                     my_lds + ((R + f) * T + t) * kTileBytes + u * 1024);
+                }
+            }
+        }
+    }
+
+    // ---- fragment layout: lane l supplies row l%16 and, in step s of a tile, chunk
+    //      4*s + l/16 (32 nibbles: even ones feed one MFMA, odd ones the next).
+    const int fr = lane & 15;
+    const int fg = lane >> 4;
+    const int sw = slot_swizzle(fr);
+    v4i xg[XDMA ? 1 : T][2][FMX];
+    if (!XDMA) {
+#pragma unroll
+        for (int f = 0; f < FMX; ++f) {
+            const int xr = f * 16 + fr;
+            const uint8_t *src = X + (size_t)(xr < M ? xr : M - 1) * rowbytes + kbyte0;
+#pragma unroll
+            for (int t = 0; t < T; ++t)
+#pragma unroll
+                for (int s = 0; s < 2; ++s)
+                    xg[t][s][f] = *(const v4i *)(src + t * kTileRowBytes + (4 * s + fg) * 16);
+        }
+    }
+
+    v4i acc[R][FMX];
+#pragma unroll
+    for (int rg = 0; rg < R; ++rg)
+#pragma unroll
+        for (int f = 0; f < FMX; ++f)
+            acc[rg][f] = (v4i){0, 0, 0, 0};
+    const int himask = (int)0xF0F0F0F0u;
+
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    const uint8_t *mine = lds + wave * kWaveTiles * kTileBytes;
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            const int off = fr * kTileRowBytes + (((4 * s + fg) ^ sw) * 16);
+            v4i xlo[FMX], xhi[FMX];
+#pragma unroll
+            for (int f = 0; f < FMX; ++f) {
+                const v4i x = XDMA ? *(const v4i *)(mine + ((R + f) * T + t) * kTileBytes + off) : xg[XDMA ? 0 : t][s][f];
+                xlo[f] = (x << 4) & himask;
+                xhi[f] = x & himask;
+            }
+#pragma unroll
+            for (int rg = 0; rg < R; ++rg) {
+                const v4i w = *(const v4i *)(mine + (rg * T + t) * kTileBytes + off);
+                const v4i wlo = (w << 4) & himask;
+                const v4i whi = w & himask;
+#pragma unroll
+                for (int f = 0; f < FMX; ++f) {
+                    acc[rg][f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo, xlo[f], acc[rg][f], 0, 0, 0);
+                    acc[rg][f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi, xhi[f], acc[rg][f], 0, 0, 0);
+                }
+            }
+        }
+    }
+
+    // ---- the S partial sums of every output meet in LDS (the staging area is free now)
+    __syncthreads();
+    v4i *partial = (v4i *)lds;  // [R*FMX][waves][64]
+#pragma unroll
+    for (int rg = 0; rg < R; ++rg)
+#pragma unroll
+        for (int f = 0; f < FMX; ++f)
+            partial[((rg * FMX + f) * waves + wave) * 64 + lane] = acc[rg][f];
+    __syncthreads();
+
+    // Element e = (rg, f, lane): n = n0 + 16*rg + 4*(lane/16) + 0..3, m = 16*f + lane%16.
+    for (int e = threadIdx.x; e < R * FMX * 64; e += blockDim.x) {
+        const int q = e >> 6, l = e & 63;
+        const v4i *p = partial + (size_t)q * waves * 64 + l;
+        v4i s = p[0];
+        for (int wv = 1; wv < waves; ++wv)
+            s += p[wv * 64];
+        s = s >> 8;  // both operands carried a factor 16
+        const int m = (q % FMX) * 16 + (l & 15);
+        const int n = n0 + (q / FMX) * 16 + 4 * (l >> 4);
+        if (m < M) {
+            int32_t *dst = Y + (size_t)m * N + n;
+            if (n + 3 < N && (N & 3) == 0) {
+                *(v4i *)dst = s;
+            } else {
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    if (n + t < N)
+                        dst[t] = s[t];
+            }
+        }
+    }
+}
+
+// ---- fallback for K that is a multiple of 128 but does not split into tiles: the
+//      straightforward version (fragment-layout global loads, 128 nibbles per step).
 template <int FMX, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void skinny_kernel(
+__global__ __launch_bounds__(WAVES * 64) void skinny_basic_kernel(
     const uint8_t *__restrict__ X, const uint8_t *__restrict__ W, int32_t *__restrict__ Y,
     int M, int N, int K)
 {
     __shared__ v4i partial[WAVES][FMX][64];
-
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int fr = lane & 15;  // operand row inside a 16-row fragment
-    const int fg = lane >> 4;  // which 16-byte quarter of the 64-byte step
+    const int fr = lane & 15;
+    const int fg = lane >> 4;
     const int rowbytes = K >> 1;
-    const int KT = K / kStepK;
+    const int KT = K / 128;
     const int n0 = blockIdx.x * 16;
-
     const int wrow = (n0 + fr < N) ? n0 + fr : N - 1;
     const uint8_t *wp = W + (size_t)wrow * rowbytes + fg * 16;
     const uint8_t *xp[FMX];
@@ -45,64 +218,34 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(
         const int xrow = (f * 16 + fr < M) ? f * 16 + fr : M - 1;
         xp[f] = X + (size_t)xrow * rowbytes + fg * 16;
     }
-
     const int himask = (int)0xF0F0F0F0u;
     v4i acc[FMX];
 #pragma unroll
     for (int f = 0; f < FMX; ++f)
         acc[f] = (v4i){0, 0, 0, 0};
-
-    auto mac = [&](const v4i &w, const v4i (&x)[FMX]) {
+    for (int ks = wave; ks < KT; ks += WAVES) {
+        const size_t off = (size_t)ks * 64;
+        const v4i w = __builtin_nontemporal_load((const v4i *)(wp + off));
         const v4i wlo = (w << 4) & himask;
         const v4i whi = w & himask;
 #pragma unroll
         for (int f = 0; f < FMX; ++f) {
-            const v4i xlo = (x[f] << 4) & himask;
-            const v4i xhi = x[f] & himask;
-            acc[f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo, xlo, acc[f], 0, 0, 0);
-            acc[f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi, xhi, acc[f], 0, 0, 0);
+            const v4i x = *(const v4i *)(xp[f] + off);
+            acc[f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo, (x << 4) & himask, acc[f], 0, 0, 0);
+            acc[f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi, x & himask, acc[f], 0, 0, 0);
         }
-    };
-
-    int ks = wave;
-    // Full batches: all loads of kBatch steps are in flight before the first use.
-    for (; ks + (kBatch - 1) * WAVES < KT; ks += kBatch * WAVES) {
-        v4i w[kBatch], x[kBatch][FMX];
-#pragma unroll
-        for (int u = 0; u < kBatch; ++u) {
-            const size_t off = (size_t)(ks + u * WAVES) * kStepBytes;
-            w[u] = __builtin_nontemporal_load((const v4i *)(wp + off));
-#pragma unroll
-            for (int f = 0; f < FMX; ++f)
-                x[u][f] = *(const v4i *)(xp[f] + off);
-        }
-#pragma unroll
-        for (int u = 0; u < kBatch; ++u)
-            mac(w[u], x[u]);
     }
-    for (; ks < KT; ks += WAVES) {
-        const size_t off = (size_t)ks * kStepBytes;
-        v4i w = __builtin_nontemporal_load((const v4i *)(wp + off));
-        v4i x[FMX];
-#pragma unroll
-        for (int f = 0; f < FMX; ++f)
-            x[f] = *(const v4i *)(xp[f] + off);
-        mac(w, x);
-    }
-
 #pragma unroll
     for (int f = 0; f < FMX; ++f)
         partial[wave][f][lane] = acc[f];
     __syncthreads();
-
-    // Element e = (f, lane): n = n0 + 4*(lane/16) + 0..3, m = f*16 + lane%16.
     for (int e = threadIdx.x; e < FMX * 64; e += WAVES * 64) {
         const int f = e >> 6, l = e & 63;
         v4i s = partial[0][f][l];
 #pragma unroll
         for (int wv = 1; wv < WAVES; ++wv)
             s += partial[wv][f][l];
-        s = s >> 8;  // both operands carried a factor 16
+        s = s >> 8;
         const int m = f * 16 + (l & 15);
         const int n = n0 + 4 * (l >> 4);
         if (m < M) {
@@ -119,63 +262,161 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(
     }
 }
 
-template <int FMX, int WAVES>
-hipError_t launch_one(const void *a, const void *b, void *c, int m, int n, int k,
-                      hipStream_t stream)
+template <int FMX>
+hipError_t launch_basic(const void *a, const void *b, void *c, int m, int n, int k,
+                        hipStream_t stream)
 {
     const unsigned grid = (unsigned)((n + 15) / 16);
-    skinny_kernel<FMX, WAVES><<<grid, WAVES * 64, 0, stream>>>(
-        (const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k);
+    const int steps = k / 128;
+    if (steps >= 8)
+        skinny_basic_kernel<FMX, 8><<<grid, 512, 0, stream>>>((const uint8_t *)a, (const uint8_t *)b,
+                                                              (int32_t *)c, m, n, k);
+    else
+        skinny_basic_kernel<FMX, 2><<<grid, 128, 0, stream>>>((const uint8_t *)a, (const uint8_t *)b,
+                                                              (int32_t *)c, m, n, k);
     return hipGetLastError();
 }
 
-template <int WAVES>
-hipError_t launch_fmx(const void *a, const void *b, void *c, int m, int n, int k,
-                      hipStream_t stream)
+struct Plan {
+    int t = 0, s = 0, r = 0, fmx = 0;
+    bool xdma = true;
+    int lds = 0;
+};
+
+// Largest S <= 16 with S * T == tiles for the smallest T <= 4; R as large as keeps
+// R * FMX <= 4, the grid near the CU count and the staging inside LDS.
+bool make_plan(int m, int n, int k, int cu_count, Plan &p)
 {
-    switch ((m + 15) / 16) {
-    case 1:
-        return launch_one<1, WAVES>(a, b, c, m, n, k, stream);
-    case 2:
-        return launch_one<2, WAVES>(a, b, c, m, n, k, stream);
-    case 3:
-        return launch_one<3, WAVES>(a, b, c, m, n, k, stream);
-    default:
-        return launch_one<4, WAVES>(a, b, c, m, n, k, stream);
+    if (k % kTileK != 0)
+        return false;
+    const int tiles = k / kTileK;
+    p.fmx = (m + 15) / 16;
+    p.t = 0;
+    for (int t = 1; t <= 4; ++t)
+        if (tiles % t == 0 && tiles / t <= 16) {
+            p.t = t;
+            p.s = tiles / t;
+            break;
+        }
+    if (p.t == 0)
+        return false;
+    auto lds_for = [&](int r, bool xdma) {
+        const int staging = p.s * p.t * (r + (xdma ? p.fmx : 0)) * kTileBytes;
+        const int reduce = r * p.fmx * p.s * 1024;
+        return staging > reduce ? staging : reduce;
+    };
+    for (int r = 4; r >= 1; r >>= 1) {
+        if (r * p.fmx > 4)
+            continue;
+        const long blocks = (n + 16 * r - 1) / (16 * r);
+        if (r > 1 && blocks * 10 < (long)cu_count * 8)
+            continue;  // too few workgroups: prefer smaller R
+        for (int xd = 1; xd >= 0; --xd) {
+            if (xd == 0 && (p.t != 4 || p.fmx > 2))
+                continue;  // the register-X variant exists for T == 4, M <= 32 only
+            if (lds_for(r, xd != 0) <= kMaxLds) {
+                p.r = r;
+                p.xdma = xd != 0;
+                p.lds = lds_for(r, p.xdma);
+                return true;
+            }
+        }
     }
+    return false;
+}
+
+template <int T, int R, int FMX, bool XDMA>
+hipError_t launch_plan(const Plan &p, const void *a, const void *b, void *c, int m, int n, int k,
+                       hipStream_t stream)
+{
+    if constexpr (!XDMA && FMX > 2) {
+        return p.s == 0 ? hipSuccess : hipErrorInvalidConfiguration;  // never planned
+    } else {
+    auto kern = skinny_kernel<T, R, FMX, XDMA>;
+    if (p.s == 0)  // set-up call: raise the dynamic-LDS limit of this instantiation
+        return hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
+    const unsigned grid = (unsigned)((n + 16 * R - 1) / (16 * R));
+    kern<<<grid, p.s * 64, p.lds, stream>>>((const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k);
+    return hipGetLastError();
+    }
+}
+
+template <int T, bool XDMA>
+hipError_t dispatch_rf(const Plan &p, const void *a, const void *b, void *c, int m, int n, int k,
+                       hipStream_t stream)
+{
+#define I4L_CASE(R_, F_)                                                      \
+    if (p.r == R_ && p.fmx == F_)                                             \
+        return launch_plan<T, R_, F_, XDMA>(p, a, b, c, m, n, k, stream);
+    I4L_CASE(4, 1)
+    I4L_CASE(2, 1)
+    I4L_CASE(1, 1)
+    I4L_CASE(2, 2)
+    I4L_CASE(1, 2)
+    I4L_CASE(1, 3)
+    I4L_CASE(1, 4)
+#undef I4L_CASE
+    return hipErrorInvalidConfiguration;
 }
 
 }  // namespace
 
+hipError_t skinny_init(const DeviceInfo &)
+{
+    // Every instantiation may use up to the full LDS of a CU.
+    static const int kRf[7][2] = {{4, 1}, {2, 1}, {1, 1}, {2, 2}, {1, 2}, {1, 3}, {1, 4}};
+    for (const auto &rf : kRf) {
+        Plan p;
+        p.s = 0;
+        p.r = rf[0];
+        p.fmx = rf[1];
+        hipError_t e = dispatch_rf<1, true>(p, nullptr, nullptr, nullptr, 0, 0, 0, nullptr);
+        if (e == hipSuccess)
+            e = dispatch_rf<2, true>(p, nullptr, nullptr, nullptr, 0, 0, 0, nullptr);
+        if (e == hipSuccess)
+            e = dispatch_rf<3, true>(p, nullptr, nullptr, nullptr, 0, 0, 0, nullptr);
+        if (e == hipSuccess)
+            e = dispatch_rf<4, true>(p, nullptr, nullptr, nullptr, 0, 0, 0, nullptr);
+        if (e == hipSuccess)
+            e = dispatch_rf<4, false>(p, nullptr, nullptr, nullptr, 0, 0, 0, nullptr);
+        if (e != hipSuccess)
+            return e;
+    }
+    return hipSuccess;
+}
+
 bool skinny_supports(int m, int n, int k)
 {
-    return m >= 1 && m <= 64 && n >= 1 && k >= kStepK && k % kStepK == 0 && k <= 131071 - 127;
+    return m >= 1 && m <= 64 && n >= 1 && k >= 128 && k % 128 == 0 && k <= 131071 - 127;
 }
 
 hipError_t launch_skinny(const void *a, const void *b, void *c, int m, int n, int k,
                          const DeviceInfo &dev, hipStream_t stream)
 {
-    // Wavefronts per workgroup: enough K-splitting that the grid fills the device with
-    // at least ~8 waves per CU, bounded by the number of K steps.
-    const long groups = (n + 15) / 16;
-    const int steps = k / kStepK;
-    const long want_waves = (long)dev.cu_count * 8;
-    int waves = 4;
-    while (waves < 16 && groups * waves < want_waves && waves * 2 <= steps)
-        waves *= 2;
-    if (waves > steps)
-        waves = steps >= 8 ? 8 : (steps >= 4 ? 4 : (steps >= 2 ? 2 : 1));
-    switch (waves) {
+    Plan p;
+    if (make_plan(m, n, k, dev.cu_count, p)) {
+        if (!p.xdma)
+            return dispatch_rf<4, false>(p, a, b, c, m, n, k, stream);
+        switch (p.t) {
+        case 1:
+            return dispatch_rf<1, true>(p, a, b, c, m, n, k, stream);
+        case 2:
+            return dispatch_rf<2, true>(p, a, b, c, m, n, k, stream);
+        case 3:
+            return dispatch_rf<3, true>(p, a, b, c, m, n, k, stream);
+        default:
+            return dispatch_rf<4, true>(p, a, b, c, m, n, k, stream);
+        }
+    }
+    switch ((m + 15) / 16) {
     case 1:
-        return launch_fmx<1>(a, b, c, m, n, k, stream);
+        return launch_basic<1>(a, b, c, m, n, k, stream);
     case 2:
-        return launch_fmx<2>(a, b, c, m, n, k, stream);
-    case 4:
-        return launch_fmx<4>(a, b, c, m, n, k, stream);
-    case 8:
-        return launch_fmx<8>(a, b, c, m, n, k, stream);
+        return launch_basic<2>(a, b, c, m, n, k, stream);
+    case 3:
+        return launch_basic<3>(a, b, c, m, n, k, stream);
     default:
-        return launch_fmx<16>(a, b, c, m, n, k, stream);
+        return launch_basic<4>(a, b, c, m, n, k, stream);
     }
 }
 

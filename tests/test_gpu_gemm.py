@@ -94,6 +94,26 @@ def test_cfg4_decode(gpu, host_threads, m, n, k):
         assert np.array_equal(got, want), f"kernel={kern}"
 
 
+# Every plan family of the weight-streaming kernel: tiles per wave 1..4, 1/2/4 row groups
+# per workgroup (chosen from N against the CU count), 1..4 sixteen-row groups of X, the
+# register-X variant (K = 14336), the fallback for K % 256 != 0 and for very long K.
+@pytest.mark.parametrize("m, n, k", [
+    (1, 5, 256), (7, 100, 512), (16, 4099, 768), (17, 7000, 1024), (33, 6600, 2048), (48, 333, 4096),
+    (64, 4096, 8192), (16, 13200, 8192), (5, 6560, 12288), (32, 6556, 12288), (64, 1030, 16384),
+    (16, 13112, 14336), (32, 6562, 14336), (40, 515, 14336), (9, 1000, 1920), (64, 200, 20480),
+    (16, 14336, 4096 + 256), (3, 16, 4096),
+])
+def test_skinny_plans(gpu, host_threads, m, n, k):
+    x = helpers.normal_s4(500 + m + k, m, k)
+    w = helpers.uniform_s4(600 + n + k, n, k)
+    want = oracle.linear_ref(x, w, threads=host_threads)
+    xp, wp = helpers.pack_bytes(x), helpers.pack_bytes(w)
+    for kern in ("skinny", "auto"):
+        got = helpers.run_gemm(xp, wp, m, n, k, kernel=kern)
+        bad = np.argwhere(got != want)
+        assert bad.size == 0, f"kernel={kern}: {len(bad)} mismatches, first at {tuple(bad[0])}"
+
+
 # ---- configuration 5: adversarial ---------------------------------------------------------
 
 def test_cfg5_all_minus_eight_full_size(gpu):
