@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the packed-int4 linear-layer GEMM on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-decode]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-decode] [--calibrate-copy]
 
 A step is one GEMM launch C[MxN] = A[MxK] * B[NxK]^T through the library's C ABI
 (int4linear_gemm_s4s4s32, asynchronous, on torch's current stream).  The workload is
@@ -12,8 +12,9 @@ operands cached by the previous one (the reference flushes L2 before every timed
 test/benchmark.cu:77-96).  Throughput = 2*M*N*K / time (test/benchmark.cu:112-115).
 
 One JSON line is printed.  Besides the whole-run figure it carries
-  roofline      the GEMM kernel's own rate (HIP events around the timed launches on the
-                launch stream) against the int8 MFMA dense peak,
+  roofline      the dominant kernel's own rate (HIP events around launches of the GEMM
+                kernel alone, on the launch stream) against the dense peak of the MFMA
+                type it issues,
   decode        the skinny-M weight-streaming kernel at M = 16 against HBM bandwidth,
   cpu_baseline  the CPU oracle's loop nest timed on this host's cores on a row sample.
 """
@@ -32,6 +33,7 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 INT8_MFMA_PEAK_TOPS = 5000.0   # MI355X dense int8, published
+FP6_MFMA_PEAK_TOPS = 10100.0   # MI355X dense fp6/fp4, published
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 
 M = N = K = 8192
@@ -64,7 +66,18 @@ def time_launches(torch, launch, sets, steps: int, warmup: int):
     return start.elapsed_time(stop) / steps, wall_ms / steps
 
 
+def raw_entry(name: str):
+    """The C-ABI function itself (ctypes), so the timed loops carry no wrapper overhead."""
+    from int4linear_amd import _lib
+
+    return getattr(_lib.load(), name)
+
+
 def bench_gemm(torch, lib, steps: int, warmup: int):
+    """The drop-in call (packed s4 in, int32 out) and, separately, its dominant kernel."""
+    import ctypes
+
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     # 3 operand sets x (32 + 32 + 256 MiB) = 960 MiB > L2 + Infinity Cache.
     sets = []
     for s in range(3):
@@ -72,15 +85,44 @@ def bench_gemm(torch, lib, steps: int, warmup: int):
         b = packed_random(torch, N, K, 2000 + s)
         c = torch.empty((M, N), dtype=torch.int32, device="cuda")
         sets.append((a, b, c))
+    gemm = raw_entry("int4linear_gemm_s4s4s32")
+    args = [(a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K, stream) for (a, b, c) in sets]
 
     def launch(t):
-        lib.gemm_s4s4s32(t[0], t[1], t[2], M, N, K)
+        st = gemm(*t)
+        if st != 0:
+            raise RuntimeError(f"int4linear_gemm_s4s4s32 failed with status {st}")
 
-    ev_ms, wall_ms = time_launches(torch, launch, sets, steps, warmup)
-    return ev_ms, wall_ms
+    ev_ms, wall_ms = time_launches(torch, launch, args, steps, warmup)
+
+    # The dominant kernel alone: the FP6 GEMM on operands converted beforehand.
+    kernel = lib.kernel_for_shape(M, N, K)
+    kern_ms = ev_ms
+    if kernel == "fp6":
+        conv = []
+        for (a, b, c) in sets:
+            ac = torch.empty(lib.fp6_operand_bytes(M, K), dtype=torch.uint8, device="cuda")
+            bc = torch.empty(lib.fp6_operand_bytes(N, K), dtype=torch.uint8, device="cuda")
+            lib.fp6_convert(a, ac, M, K)
+            lib.fp6_convert(b, bc, N, K)
+            conv.append((ac, bc, c))
+        gemm6 = raw_entry("int4linear_gemm_fp6_converted")
+        args6 = [(a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K, stream) for (a, b, c) in conv]
+
+        def launch6(t):
+            st = gemm6(*t)
+            if st != 0:
+                raise RuntimeError(f"int4linear_gemm_fp6_converted failed with status {st}")
+
+        kern_ms, _ = time_launches(torch, launch6, args6, steps, warmup)
+    return ev_ms, wall_ms, kernel, kern_ms
 
 
 def bench_decode(torch, lib, steps: int, warmup: int):
+    import ctypes
+
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    gemm = raw_entry("int4linear_gemm_s4s4s32")
     out = []
     for (m, n, k) in DECODE_SHAPES:
         wbytes = n * k // 2
@@ -88,11 +130,14 @@ def bench_decode(torch, lib, steps: int, warmup: int):
         x = packed_random(torch, m, k, 31)
         sets = [(x, packed_random(torch, n, k, 40 + i), torch.empty((m, n), dtype=torch.int32, device="cuda"))
                 for i in range(nsets)]
+        args = [(a.data_ptr(), b.data_ptr(), c.data_ptr(), m, n, k, stream) for (a, b, c) in sets]
 
-        def launch(t, m=m, n=n, k=k):
-            lib.gemm_s4s4s32(t[0], t[1], t[2], m, n, k)
+        def launch(t):
+            st = gemm(*t)
+            if st != 0:
+                raise RuntimeError(f"int4linear_gemm_s4s4s32 failed with status {st}")
 
-        ev_ms, _ = time_launches(torch, launch, sets, max(steps, 200), max(warmup, 20))
+        ev_ms, _ = time_launches(torch, launch, args, max(steps, 300), max(warmup, 20))
         algo_bytes = m * k // 2 + n * k // 2 + 4 * m * n
         gbs = algo_bytes / (ev_ms * 1e-3) / 1e9
         out.append({"shape": [m, n, k], "kernel": lib.kernel_for_shape(m, n, k), "us_per_launch": ev_ms * 1e3,
@@ -102,7 +147,7 @@ def bench_decode(torch, lib, steps: int, warmup: int):
     return out
 
 
-def cpu_baseline(budget_s: float = 12.0):
+def cpu_baseline(budget_s: float = 15.0):
     """The oracle's loop nest (oracle_linear_ref_mt) on a row sample of the 8192^3
     problem, all host threads the box grants us."""
     from oracle import loader as oracle
@@ -127,14 +172,17 @@ def cpu_baseline(budget_s: float = 12.0):
                       f"{dt:.1f} s, oracle_linear_ref_mt with {threads} threads"}
 
 
-def measured_traffic():
-    """HBM bytes per launch of the GEMM kernel from rocprofv3 counter runs, if recorded."""
-    f = ROOT / "profiles" / "traffic.json"
+def measured_traffic(kernel: str):
+    """HBM bytes per launch of the GEMM kernel as recorded from rocprofv3 counter runs
+    (FETCH_SIZE and WRITE_SIZE, each scaled by a plain copy of known size), or None."""
+    f = ROOT / "profiles" / "bench_default_hbm_traffic.md"
     if f.exists():
-        try:
-            return json.loads(f.read_text()).get("mfma_gemm_8192", {}).get("bytes_per_launch")
-        except Exception:
-            return None
+        for line in f.read_text().splitlines():
+            if line.startswith(f"bytes_per_launch {kernel}_gemm_8192:"):
+                try:
+                    return int(line.split(":")[1])
+                except ValueError:
+                    return None
     return None
 
 
@@ -145,6 +193,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="skip the decode-shape leg")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run four plain 1 GiB device copies first (a kernel of known traffic "
+                         "to scale hardware byte counters by when profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only; run with --gpus 1 "
@@ -161,10 +212,23 @@ def main() -> int:
     lib.init()
     torch.cuda.set_device(0)
 
-    ev_ms, wall_ms = bench_gemm(torch, lib, args.steps, args.warmup)
+    if args.calibrate_copy:
+        src = torch.zeros(1 << 30, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
+
+    ev_ms, wall_ms, kernel, kern_ms = bench_gemm(torch, lib, args.steps, args.warmup)
     ops = 2.0 * M * N * K
-    tops_kernel = ops / (ev_ms * 1e-3) / 1e12
+    tops_kernel = ops / (kern_ms * 1e-3) / 1e12
     tops_wall = ops / (wall_ms * 1e-3) / 1e12
+    # The roofline that bounds the dominant kernel is that of the MFMA type it issues.
+    peak = FP6_MFMA_PEAK_TOPS if kernel == "fp6" else INT8_MFMA_PEAK_TOPS
+    kernel_name = {"fp6": "fp6_gemm_kernel (v_mfma_scale_f32_32x32x64_f8f6f4, E2M3 operands)",
+                   "mfma": "mfma_gemm_kernel (v_mfma_i32_32x32x32_i8)"}.get(kernel, kernel)
 
     result = {
         "metric": "INT4 GEMM TOPS at M=N=K=8192 (% int8 MFMA peak); GB/s at M=16 decode",
@@ -177,16 +241,19 @@ def main() -> int:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "int8",
+        "dtype": "fp6-e2m3 operands, fp32 accumulate (exact integers)" if kernel == "fp6" else "int8",
         "data": "synthetic",
         "config": {"workload": "M=N=K=8192 s4*s4->s32 GEMM, uniform [-8,7], 3 rotating operand sets",
-                   "kernel": lib.kernel_for_shape(M, N, K), "M": M, "N": N, "K": K},
+                   "kernel": kernel, "M": M, "N": N, "K": K},
         "pct_of_int8_mfma_peak": 100.0 * tops_wall / INT8_MFMA_PEAK_TOPS,
-        "roofline": {"bound": "mfma", "achieved": tops_kernel, "peak": INT8_MFMA_PEAK_TOPS,
-                     "unit": "TFLOP/s", "frac": tops_kernel / INT8_MFMA_PEAK_TOPS,
-                     "traffic": measured_traffic(),
-                     "note": "integer ops: 2*M*N*K per launch / mean launch time (HIP events)",
-                     "kernel_ms": ev_ms},
+        "roofline": {"bound": "mfma", "achieved": tops_kernel, "peak": peak,
+                     "unit": "TFLOP/s", "frac": tops_kernel / peak,
+                     "traffic": measured_traffic(kernel),
+                     "kernel": kernel_name,
+                     "note": "2*M*N*K multiply-adds per launch / mean duration of the GEMM kernel alone "
+                             "(HIP events around launches on pre-converted operands)",
+                     "kernel_ms": kern_ms, "whole_call_ms": ev_ms,
+                     "frac_of_int8_peak": tops_kernel / INT8_MFMA_PEAK_TOPS},
     }
     if not args.no_decode:
         dec = bench_decode(torch, lib, args.steps, args.warmup)

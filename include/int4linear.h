@@ -43,7 +43,7 @@ enum {
 enum {
     INT4LINEAR_KERNEL_AUTO = 0,   /* shape-based dispatch (what the plain entry uses)    */
     INT4LINEAR_KERNEL_SIMPLE = 1, /* one thread per output, scalar nibble decode; any K%8==0 */
-    INT4LINEAR_KERNEL_MFMA = 2,   /* LDS-pipelined v_mfma_i32_16x16x64_i8 kernel; K%128==0 */
+    INT4LINEAR_KERNEL_MFMA = 2,   /* LDS-pipelined v_mfma_i32_32x32x32_i8 kernel; K%128==0 */
     INT4LINEAR_KERNEL_SKINNY = 3, /* weight-streaming kernel for M <= 64; K%128==0       */
     INT4LINEAR_KERNEL_FP6 = 4     /* operands converted to FP6 (E2M3) in a workspace, then
                                      v_mfma_scale_f32_32x32x64_f8f6f4; exact; K%128==0,
@@ -74,6 +74,21 @@ int int4linear_gemm_s4s4s32_ex(const void *a_packed_d, const void *b_packed_d, v
  * unpacked, m x ceil(n/8) 32-bit words packed).  Asynchronous on `stream`. */
 int int4linear_pack_s32_to_s4(const int *src_d, int *dst_d, int m, int n, void *stream);
 int int4linear_unpack_s4_to_s32(const int *src_d, int *dst_d, int m, int n, void *stream);
+
+/* The two halves of INT4LINEAR_KERNEL_FP6 on caller-owned memory, for callers whose
+ * weights are static (a linear layer converts W once when it is loaded and X per call)
+ * or who may not let the library allocate.  The reference has no counterpart: it
+ * consumes the packed layout directly (kernels/linear_v21.cu:121-172).
+ *   int4linear_fp6_operand_bytes  size of the converted form of a rows x k operand
+ *                                 (0 if the FP6 kernel cannot take this k);
+ *   int4linear_fp6_convert        packed s4 (rows x k/2 bytes) -> converted form;
+ *                                 converted_d must be 256-byte aligned;
+ *   int4linear_gemm_fp6_converted C = A * B^T from two converted operands.
+ * The converted form is opaque and specific to this library version. */
+size_t int4linear_fp6_operand_bytes(int rows, int k);
+int int4linear_fp6_convert(const void *packed_d, void *converted_d, int rows, int k, void *stream);
+int int4linear_gemm_fp6_converted(const void *a_conv_d, const void *b_conv_d, void *c_d,
+                                  int m, int n, int k, void *stream);
 
 /* Bytes of internal workspace INT4LINEAR_KERNEL_AUTO would use for a shape (0 when the
  * chosen kernel needs none). */

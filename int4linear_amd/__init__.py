@@ -5,6 +5,9 @@ The compute lives in ``lib/libint4linear.so`` (HIP kernels + C ABI, declared in
 ``linear_vN_launch`` / ``pack`` / ``unpack`` interface.
 """
 from .api import (  # noqa: F401
+    fp6_convert,
+    fp6_operand_bytes,
+    gemm_fp6_converted,
     gemm_s4s4s32,
     init,
     kernel_for_shape,

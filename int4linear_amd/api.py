@@ -51,6 +51,28 @@ def gemm_s4s4s32(a_packed_d, b_packed_d, c_d, m: int, n: int, k: int, *, kernel:
     _lib.check(st)
 
 
+def fp6_operand_bytes(rows: int, k: int) -> int:
+    """Bytes of the converted (FP6) form of a rows x k operand; 0 if k is unsupported."""
+    return int(_lib.load().int4linear_fp6_operand_bytes(rows, k))
+
+
+def fp6_convert(packed_d, converted_d, rows: int, k: int, *, stream: int | None = None) -> None:
+    """Packed s4 operand -> the FP6 kernel's own operand form (convert static weights once)."""
+    lib = _lib.load()
+    if stream is None:
+        stream = _current_stream()
+    _lib.check(lib.int4linear_fp6_convert(_ptr(packed_d), _ptr(converted_d), rows, k, ctypes.c_void_p(stream)))
+
+
+def gemm_fp6_converted(a_conv_d, b_conv_d, c_d, m: int, n: int, k: int, *, stream: int | None = None) -> None:
+    """C = A * B^T from two operands already converted with fp6_convert."""
+    lib = _lib.load()
+    if stream is None:
+        stream = _current_stream()
+    _lib.check(lib.int4linear_gemm_fp6_converted(_ptr(a_conv_d), _ptr(b_conv_d), _ptr(c_d), m, n, k,
+                                                 ctypes.c_void_p(stream)))
+
+
 def workspace_bytes(m: int, n: int, k: int) -> int:
     """Internal workspace the automatic dispatch would use for this shape."""
     return int(_lib.load().int4linear_workspace_bytes(m, n, k))

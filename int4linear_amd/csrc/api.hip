@@ -276,6 +276,53 @@ int int4linear_unpack_s4_to_s32(const int *src_d, int *dst_d, int m, int n, void
     return e == hipSuccess ? INT4LINEAR_OK : fail_hip(e);
 }
 
+size_t int4linear_fp6_operand_bytes(int rows, int k)
+{
+    if (rows <= 0 || !fp6_supports(rows, 1, k))
+        return 0;
+    return fp6_operand_bytes(rows, k);
+}
+
+int int4linear_fp6_convert(const void *packed_d, void *converted_d, int rows, int k, void *stream)
+{
+    if (rows < 0 || k < 0 || (k % 8) != 0)
+        return INT4LINEAR_ERR_SHAPE;
+    if (rows == 0)
+        return INT4LINEAR_OK;
+    if (!fp6_supports(rows, 1, k))
+        return INT4LINEAR_ERR_UNSUPPORTED;
+    if (!packed_d || !converted_d)
+        return INT4LINEAR_ERR_NULL;
+    if (!aligned16(packed_d) || ((uintptr_t)converted_d & 255) != 0)
+        return INT4LINEAR_ERR_ALIGN;
+    int st = ensure_init(nullptr);
+    if (st != INT4LINEAR_OK)
+        return st;
+    hipError_t e = launch_fp6_convert(packed_d, converted_d, rows, k, (hipStream_t)stream);
+    return e == hipSuccess ? INT4LINEAR_OK : fail_hip(e);
+}
+
+int int4linear_gemm_fp6_converted(const void *a_conv_d, const void *b_conv_d, void *c_d, int m, int n,
+                                  int k, void *stream)
+{
+    if (m < 0 || n < 0 || k < 0 || (k % 8) != 0)
+        return INT4LINEAR_ERR_SHAPE;
+    if (m == 0 || n == 0)
+        return INT4LINEAR_OK;
+    if (!fp6_supports(m, n, k))
+        return INT4LINEAR_ERR_UNSUPPORTED;
+    if (!a_conv_d || !b_conv_d || !c_d)
+        return INT4LINEAR_ERR_NULL;
+    if (!aligned16(c_d) || ((uintptr_t)a_conv_d & 255) != 0 || ((uintptr_t)b_conv_d & 255) != 0)
+        return INT4LINEAR_ERR_ALIGN;
+    PerDevice *pd = nullptr;
+    int st = ensure_init(&pd);
+    if (st != INT4LINEAR_OK)
+        return st;
+    hipError_t e = launch_fp6_gemm(a_conv_d, b_conv_d, c_d, m, n, k, pd->info, (hipStream_t)stream);
+    return e == hipSuccess ? INT4LINEAR_OK : fail_hip(e);
+}
+
 const char *int4linear_kernel_for_shape(int m, int n, int k)
 {
     if (m < 0 || n < 0 || k < 0 || (k % 8) != 0)

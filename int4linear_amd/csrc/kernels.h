@@ -26,6 +26,12 @@ hipError_t launch_mfma(const void *a, const void *b, void *c, int m, int n, int 
 bool fp6_supports(int m, int n, int k);
 size_t fp6_workspace_bytes(int m, int n, int k);
 hipError_t fp6_init(const DeviceInfo &dev);
+// The two halves of launch_fp6 on caller-owned buffers: an operand of `rows` rows converts
+// into fp6_operand_bytes(rows, k) bytes (256-byte aligned); the GEMM runs on two of those.
+size_t fp6_operand_bytes(int rows, int k);
+hipError_t launch_fp6_convert(const void *src, void *dst, int rows, int k, hipStream_t stream);
+hipError_t launch_fp6_gemm(const void *a_conv, const void *b_conv, void *c, int m, int n, int k,
+                           const DeviceInfo &dev, hipStream_t stream);
 hipError_t launch_fp6(const void *a, const void *b, void *c, int m, int n, int k, void *workspace,
                       const DeviceInfo &dev, hipStream_t stream);
 

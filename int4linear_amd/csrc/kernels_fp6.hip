@@ -261,14 +261,6 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
     const unsigned w_rd = (unsigned)(kOperandStageBytes + wn * C::FN * kFragBytes) + lane16;
     const unsigned hi_delta = (unsigned)kFragLoBytes - (unsigned)lane * 8u;  // from the 16-B to the 8-B part
 
-#ifdef I4L_EXP_TRACE
-    long long *trace = (long long *)(lds + kLdsBytes);
-    int trace_n = 0;
-    const bool tracer = (bid == 0) && (threadIdx.x == I4L_EXP_TRACE * 64);
-#define I4L_STAMP() do { if (tracer && trace_n < 1900) { trace[trace_n++] = __builtin_readcyclecounter(); } } while (0)
-#else
-#define I4L_STAMP() do {} while (0)
-#endif
     v16f acc[C::FN][C::FM];
     v4i xlo[2][C::FM], wlo[2][C::FN];  // first 128 bits of each fragment's 192
     v2i xhi[2][C::FM], whi[2][C::FN];  // last 64 bits
@@ -341,7 +333,6 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
 
 #pragma unroll 1
     for (int gs = 0; gs < total_stages; ++gs) {
-        I4L_STAMP();
         if (kk == 0) {
 #pragma unroll
             for (int i = 0; i < C::FN; ++i)
@@ -365,16 +356,13 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
         //      normally one younger stage (gs+2) is in flight behind it, and in the first
         //      stage after a tile end that tile's C stores sit behind it as well.
         {
-            I4L_STAMP();
             if (cur_it > 0 && kk < 1) {
                 constexpr int with_stores = C::CH + C::STORES;
                 __builtin_amdgcn_s_waitcnt(I4L_WAIT_VM_LGKM0(with_stores < 63 ? with_stores : 63));
             } else {
                 __builtin_amdgcn_s_waitcnt(I4L_WAIT_VM_LGKM0(C::CH));
             }
-            I4L_STAMP();
             __builtin_amdgcn_s_barrier();
-            I4L_STAMP();
             asm volatile("" ::: "memory");
         }
 
@@ -382,8 +370,6 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
         //      multiplied into a stored tile); begins the loads of stage gs+3 into the
         //      buffer of stage gs
         unit(std::integral_constant<int, 1>{}, [&](auto slot_tag) { spread(slot_tag, gs + 1, 0, 0, 0); });
-
-        I4L_STAMP();
         ++kk;
         if (kk == KT) {
             // ---- store the tile.  X is the MFMA A operand: accumulator t of tile (i, j) is
@@ -427,16 +413,6 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
             ++cur_it;
         }
     }
-#ifdef I4L_EXP_TRACE
-    I4L_STAMP();
-    __builtin_amdgcn_s_waitcnt(0);
-    if (tracer) {
-        long long *dst = (long long *)Y;
-        dst[0] = trace_n;
-        for (int i = 0; i < trace_n; ++i)
-            dst[1 + i] = trace[i];
-    }
-#endif
 }
 
 // Eight wavefronts of 128 (m) x 64 (n), two per SIMD, one workgroup per CU.
@@ -469,45 +445,48 @@ hipError_t fp6_init(const DeviceInfo &dev)
                                hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
 }
 
-hipError_t launch_fp6(const void *a, const void *b, void *c, int m, int n, int k, void *workspace,
-                      const DeviceInfo &dev, hipStream_t stream)
+size_t fp6_operand_bytes(int rows, int k) { return operand_ws_bytes(rows, k); }
+
+hipError_t launch_fp6_convert(const void *src, void *dst, int rows, int k, hipStream_t stream)
+{
+    const int tiles = (rows + kTileRows - 1) / kTileRows;
+    if (tiles * kFragsRows > 65535)
+        return hipErrorInvalidValue;
+    // One converter workgroup per 32 rows x 256 k (K % 256 may be 128: the kernel guards).
+    const int kblocks = (k + 255) / 256;
+    fp6_convert_kernel<<<dim3(kblocks, tiles * kFragsRows), 256, 0, stream>>>(
+        (const uint8_t *)src, (uint8_t *)dst, rows, tiles * kTileRows, k);
+    return hipGetLastError();
+}
+
+hipError_t launch_fp6_gemm(const void *a_conv, const void *b_conv, void *c, int m, int n, int k,
+                           const DeviceInfo &dev, hipStream_t stream)
 {
     using C = Fp6Cfg;
-    uint8_t *xws = (uint8_t *)workspace;
-    uint8_t *wws = xws + operand_ws_bytes(m, k);
     const int tiles_m = (m + kTileRows - 1) / kTileRows;
     const int tiles_n = (n + kTileRows - 1) / kTileRows;
     const long total = (long)tiles_m * tiles_n;
     if (total > 0x7fffffffL || (size_t)kTileRows * (size_t)n * 4u > 0x40000000ull)
         return hipErrorInvalidValue;
-    if (tiles_m * 8 > 65535 || tiles_n * 8 > 65535)
-        return hipErrorInvalidValue;
-
-    // One converter workgroup per 32 rows x 256 k (K % 256 may be 128: the kernel guards).
-    const int kblocks = (k + 255) / 256;
-    fp6_convert_kernel<<<dim3(kblocks, tiles_m * kFragsRows), 256, 0, stream>>>(
-        (const uint8_t *)a, xws, m, tiles_m * kTileRows, k);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess)
-        return e;
-    fp6_convert_kernel<<<dim3(kblocks, tiles_n * kFragsRows), 256, 0, stream>>>(
-        (const uint8_t *)b, wws, n, tiles_n * kTileRows, k);
-    e = hipGetLastError();
-    if (e != hipSuccess)
-        return e;
-
     long grid = (long)dev.cu_count * C::OCC;
     if (grid > total)
         grid = total;
-#ifdef I4L_EXP_TRACE
-    hipFuncSetAttribute((const void *)fp6_gemm_kernel<C>, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes + 16000);
-    fp6_gemm_kernel<C><<<(unsigned)grid, C::THREADS, kLdsBytes + 16000, stream>>>(
-        xws, wws, (int32_t *)c, m, n, k, tiles_m, tiles_n);
-    return hipGetLastError();
-#endif
     fp6_gemm_kernel<C><<<(unsigned)grid, C::THREADS, kLdsBytes, stream>>>(
-        xws, wws, (int32_t *)c, m, n, k, tiles_m, tiles_n);
+        (const uint8_t *)a_conv, (const uint8_t *)b_conv, (int32_t *)c, m, n, k, tiles_m, tiles_n);
     return hipGetLastError();
+}
+
+hipError_t launch_fp6(const void *a, const void *b, void *c, int m, int n, int k, void *workspace,
+                      const DeviceInfo &dev, hipStream_t stream)
+{
+    uint8_t *xws = (uint8_t *)workspace;
+    uint8_t *wws = xws + operand_ws_bytes(m, k);
+    hipError_t e = launch_fp6_convert(a, xws, m, k, stream);
+    if (e == hipSuccess)
+        e = launch_fp6_convert(b, wws, n, k, stream);
+    if (e == hipSuccess)
+        e = launch_fp6_gemm(xws, wws, c, m, n, k, dev, stream);
+    return e;
 }
 
 }  // namespace int4linear

@@ -181,9 +181,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
         const unsigned dst = lds_base + buf * C::STAGE_BYTES;
         const bool is_x = c < C::X_CH;
         const int ci = (is_x ? c : c - C::X_CH) * C::NWAVES + wave;
-#ifndef I4L_EXP_NODMA
         dma16(is_x ? xptr : wptr, voff[c], dst + (is_x ? 0 : C::BM * kRowBytes) + ci * kChunkBytes);
-#endif
     };
     auto ld_advance = [&]() {
         ++issued;
@@ -236,21 +234,6 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
     //   step (u, j) widens X fragment j+1 (or fragment 0 of unit u+1) and, for j >= 1,
     //   a third of unit u+1's W fragments; step (u, 0) issues the LDS reads of unit u+1.
     // __builtin_amdgcn_sched_barrier(0) after each slot pins that order.
-#ifdef I4L_EXP_TRACE
-    long long *trace = (long long *)(lds + C::LDS_BYTES);
-    int trace_n = 0;
-    const bool tracer = (bid == I4L_EXP_TRACE) && (threadIdx.x == I4L_EXP_TRACE_WAVE * 64);
-#ifdef I4L_EXP_TRACE_STEPS
-#define I4L_STAMP() do {} while (0)
-#define I4L_STAMP2() do { if (tracer && trace_n < 3900) { trace[trace_n++] = __builtin_readcyclecounter(); } } while (0)
-#else
-#define I4L_STAMP() do { if (tracer && trace_n < 3900) { trace[trace_n++] = __builtin_readcyclecounter(); } } while (0)
-#define I4L_STAMP2() do {} while (0)
-#endif
-#else
-#define I4L_STAMP2() do {} while (0)
-#define I4L_STAMP() do {} while (0)
-#endif
     v16i acc[C::FN][C::FM];
     v4i pk_w[2][C::FN], pk_x[2][C::FM];  // packed fragments, by unit parity (= half)
     v4i wlo[2][C::FN], whi[2][C::FN];    // widened W, by unit parity
@@ -280,10 +263,6 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
     // Op k (0..11) of widening one packed fragment: per dword d = k/3 a shift, its mask
     // (even-k nibbles) and the mask of the unshifted word (odd-k nibbles).
     auto widen_op = [&](int k, const v4i &p, v4i &lo, v4i &hi) {
-#ifdef I4L_EXP_NOVALU
-        if (k == 0) { lo = p; hi = p; }
-        return;
-#endif
         const int d = k / 3;
         switch (k % 3) {
         case 0:
@@ -338,14 +317,13 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
         }(std::make_integer_sequence<int, kSlots>{});
     };
 
-    auto stamp2 = [&] { I4L_STAMP2(); };
     // All steps of the unit with parity h, then the pins that keep the operands widened
     // for the next unit inside this unit's MFMA shadow.
     auto unit = [&](auto h_tag, auto &&hook) {
         constexpr int h = decltype(h_tag)::value;
         [&]<int... J>(std::integer_sequence<int, J...>) {
             ((step(h_tag, std::integral_constant<int, J>{},
-                   J + 1 < C::FM ? pk_x[h][(J + 1) % C::FM] : pk_x[1 - h][0], hook), stamp2()), ...);
+                   J + 1 < C::FM ? pk_x[h][(J + 1) % C::FM] : pk_x[1 - h][0], hook)), ...);
         }(std::make_integer_sequence<int, C::FM>{});
 #pragma unroll
         for (int i = 0; i < C::FN; ++i) {
@@ -413,7 +391,6 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
 
 #pragma unroll 1
     for (int gs = 0; gs < total_stages; ++gs) {
-        I4L_STAMP2();
         if (kk == 0) {
 #pragma unroll
             for (int i = 0; i < C::FN; ++i)
@@ -450,7 +427,6 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
                 // of that tile sit behind them as well.  (One stage later the loads waited
                 // for were themselves issued after those stores, so the stores must be done.)
                 const int ahead = issued - 2 - gs;  // stages issued after stage gs+1
-#ifndef I4L_EXP_NOWAIT
                 if (ahead >= 1) {
                     if (cur_it > 0 && kk < 1) {
                         constexpr int with_stores = C::CH + C::STORES;
@@ -461,10 +437,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
                 } else {
                     __builtin_amdgcn_s_waitcnt(I4L_VMCNT(0));
                 }
-#endif
-#ifndef I4L_EXP_NOBARRIER
                 __builtin_amdgcn_s_barrier();
-#endif
                 asm volatile("" ::: "memory");
                 // Every wave is past its reads of stage gs-1: that buffer may be refilled.
                 loading = issued < total_stages;
@@ -512,10 +485,6 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
 #pragma unroll
                     for (int i = 0; i < C::FN; ++i) {
                         const int v = acc[i][j][t] >> 8;
-#ifdef I4L_EXP_NOSTORE
-                        if (v == 0x12345) __builtin_amdgcn_raw_buffer_store_b32((unsigned)v, rsrc, 0, 0, 0);
-                        continue;
-#endif
                         __builtin_amdgcn_raw_buffer_store_b32((unsigned)v, rsrc, row_off + col_off[i], 0, I4L_STORE_AUX);
                     }
                 }
@@ -524,16 +493,6 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
             ++cur_it;
         }
     }
-#ifdef I4L_EXP_TRACE
-    I4L_STAMP();
-    __builtin_amdgcn_s_waitcnt(0);
-    if (tracer) {
-        long long *dst = (long long *)Y;
-        dst[0] = trace_n;
-        for (int i = 0; i < trace_n; ++i)
-            dst[1 + i] = trace[i];
-    }
-#endif
 }
 
 // 256 x 256 tile, eight wavefronts of 128 (m) x 64 (n), one workgroup per CU, two
@@ -565,12 +524,6 @@ hipError_t launch_cfg(const void *a, const void *b, void *c, int m, int n, int k
     // The epilogue addresses a tile's slab of C with 32-bit byte offsets below 2^30.
     if ((size_t)C::BM * (size_t)n * 4u > 0x40000000ull)
         return hipErrorInvalidValue;
-#ifdef I4L_EXP_TRACE
-    hipFuncSetAttribute((const void *)mfma_gemm_kernel<C>, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES + 32000);
-    mfma_gemm_kernel<C><<<(unsigned)grid, C::THREADS, C::LDS_BYTES + 32000, stream>>>(
-        (const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k, tiles_m, tiles_n);
-    return hipGetLastError();
-#endif
     mfma_gemm_kernel<C><<<(unsigned)grid, C::THREADS, C::LDS_BYTES, stream>>>(
         (const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k, tiles_m, tiles_n);
     return hipGetLastError();

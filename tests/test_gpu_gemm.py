@@ -114,6 +114,30 @@ def test_skinny_plans(gpu, host_threads, m, n, k):
         assert bad.size == 0, f"kernel={kern}: {len(bad)} mismatches, first at {tuple(bad[0])}"
 
 
+@pytest.mark.parametrize("m, n, k", [(300, 520, 512), (1, 1, 128), (1024, 2048, 4096), (777, 33, 1152)])
+def test_fp6_converted_operands(gpu, host_threads, m, n, k):
+    """Weights converted once, activations per call, GEMM on caller-owned buffers."""
+    import torch
+
+    import int4linear_amd as lib
+
+    x = helpers.normal_s4(700 + m, m, k)
+    w = helpers.uniform_s4(800 + n, n, k)
+    want = oracle.linear_ref(x, w, threads=host_threads)
+    xd = helpers.to_device_bytes(helpers.pack_bytes(x))
+    wd = helpers.to_device_bytes(helpers.pack_bytes(w))
+    xc = torch.full((lib.fp6_operand_bytes(m, k),), 0xA5, dtype=torch.uint8, device="cuda")
+    wc = torch.full((lib.fp6_operand_bytes(n, k),), 0x5A, dtype=torch.uint8, device="cuda")
+    y = torch.full((m, n), 0x7BADBAD, dtype=torch.int32, device="cuda")
+    lib.fp6_convert(wd, wc, n, k)
+    for _ in range(2):  # the converted weights are reused across calls
+        lib.fp6_convert(xd, xc, m, k)
+        lib.gemm_fp6_converted(xc, wc, y, m, n, k)
+        torch.cuda.synchronize()
+        assert np.array_equal(y.cpu().numpy(), want)
+        y.fill_(-1)
+
+
 # ---- configuration 5: adversarial ---------------------------------------------------------
 
 def test_cfg5_all_minus_eight_full_size(gpu):

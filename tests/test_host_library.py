@@ -103,6 +103,11 @@ def test_workspace_accounting():
     finally:
         lib.set_workspace_limit(1 << 30)
     assert lib.kernel_for_shape(8192, 8192, 8192) == "fp6"
+    # caller-owned converted operands: rows padded to 256, 0.75 byte per element
+    assert lib.fp6_operand_bytes(8192, 8192) == 8192 * 8192 * 3 // 4
+    assert lib.fp6_operand_bytes(1, 128) == 256 * 128 * 3 // 4
+    assert lib.fp6_operand_bytes(16, 200) == 0            # K % 128 != 0
+    assert lib.fp6_operand_bytes(16, 1 << 18) == 0        # beyond the exact range
 
 
 @pytest.mark.parametrize("m, n, seed", [(1, 8, 1), (3, 10, 2), (16, 64, 3), (7, 129, 4), (64, 4096, 5)])
