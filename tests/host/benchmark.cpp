@@ -1,0 +1,102 @@
+// Benchmark harness: counterpart of the reference's test/benchmark.cu:71-115 -- 5 warm-up
+// launches, 50 timed ones, every timed launch preceded by a cache-cleaning fill and bracketed
+// by its own event pair, median reported as 2*M*N*K / t in TOPS ("[PERF] ... TOPS").
+//
+//   benchmark [--kernel auto|simple|mfma|skinny|fp6] [--iters I] [--warmup W] [--no-flush] MxNxK ...
+//
+// The reference cleans twice its L2 (benchmark.cu:77-91); an MI355X also has a 256 MiB
+// memory-side cache behind the eight L2s, so the fill here is 512 MiB.  Operand values are
+// seeded uniform s4; the harness goes through the asynchronous C ABI so that the events
+// bracket the library's device work only.
+#include "harness_common.h"
+
+using namespace harness;
+
+namespace {
+
+int kernel_id(const std::string &name)
+{
+    if (name == "auto") return INT4LINEAR_KERNEL_AUTO;
+    if (name == "simple") return INT4LINEAR_KERNEL_SIMPLE;
+    if (name == "mfma") return INT4LINEAR_KERNEL_MFMA;
+    if (name == "skinny") return INT4LINEAR_KERNEL_SKINNY;
+    if (name == "fp6") return INT4LINEAR_KERNEL_FP6;
+    return -1;
+}
+
+}  // namespace
+
+int main(int argc, char **argv)
+{
+    std::string kernel = "auto";
+    int iters = 50, warmup = 5;
+    bool flush = true;
+    std::vector<Shape> shapes;
+    for (int i = 1; i < argc; ++i) {
+        const std::string a = argv[i];
+        Shape s;
+        if (a == "--kernel" && i + 1 < argc) kernel = argv[++i];
+        else if (a == "--iters" && i + 1 < argc) iters = std::atoi(argv[++i]);
+        else if (a == "--warmup" && i + 1 < argc) warmup = std::atoi(argv[++i]);
+        else if (a == "--no-flush") flush = false;
+        else if (parse_shape(argv[i], s)) shapes.push_back(s);
+        else {
+            std::fprintf(stderr, "usage: %s [--kernel auto|simple|mfma|skinny|fp6] [--iters I] [--warmup W] "
+                                 "[--no-flush] MxNxK ...\n", argv[0]);
+            return 2;
+        }
+    }
+    const int kid = kernel_id(kernel);
+    if (kid < 0 || iters < 1) {
+        std::fprintf(stderr, "bad --kernel or --iters\n");
+        return 2;
+    }
+    if (shapes.empty()) shapes.push_back({8192, 8192, 8192});
+
+    const size_t fill_bytes = 512ull << 20;
+    DeviceBuffer fill(flush ? fill_bytes : 16);
+    hipEvent_t start, stop;
+    HIP_OK(hipEventCreate(&start));
+    HIP_OK(hipEventCreate(&stop));
+
+    for (const Shape &s : shapes) {
+        const int m = s.m, n = s.n, k = s.k;
+        const size_t packed_k = (size_t)(k + 7) / 8;
+        DeviceBuffer xd(m * packed_k * sizeof(int)), wd(n * packed_k * sizeof(int)), yd((size_t)m * n * sizeof(int));
+        upload_packed(uniform_s4(11, (size_t)m * k), m, k, xd);
+        upload_packed(uniform_s4(12, (size_t)n * k), n, k, wd);
+
+        auto launch = [&]() {
+            const int st = int4linear_gemm_s4s4s32_ex(xd.p, wd.p, yd.p, m, n, k, kid, nullptr);
+            if (st != INT4LINEAR_OK) {
+                std::fprintf(stderr, "[%dx%dx%d] %s\n", m, n, k, int4linear_status_string(st));
+                std::exit(2);
+            }
+        };
+        for (int i = 0; i < warmup; ++i) {
+            launch();
+            HIP_OK(hipDeviceSynchronize());
+        }
+        std::vector<float> ms((size_t)iters);
+        for (int i = 0; i < iters; ++i) {
+            if (flush)
+                HIP_OK(hipMemsetAsync(fill.p, i & 0xFF, fill_bytes, nullptr));
+            HIP_OK(hipDeviceSynchronize());
+            HIP_OK(hipEventRecord(start, nullptr));
+            launch();
+            HIP_OK(hipEventRecord(stop, nullptr));
+            HIP_OK(hipEventSynchronize(stop));
+            HIP_OK(hipEventElapsedTime(&ms[i], start, stop));
+        }
+        std::sort(ms.begin(), ms.end());
+        const double median_ms = ms[(size_t)iters / 2];
+        const double ops = 2.0 * m * (double)n * k;
+        const double bytes = (double)m * k / 2 + (double)n * k / 2 + 4.0 * m * n;
+        std::printf("[PERF] %dx%dx%d kernel=%s median %.4f ms (min %.4f)  %lf TOPS  %.1f GB/s\n", m, n, k,
+                    kid == INT4LINEAR_KERNEL_AUTO ? int4linear_kernel_for_shape(m, n, k) : kernel.c_str(),
+                    median_ms, (double)ms[0], ops / (median_ms * 1e9), bytes / (median_ms * 1e6));
+    }
+    HIP_OK(hipEventDestroy(start));
+    HIP_OK(hipEventDestroy(stop));
+    return 0;
+}

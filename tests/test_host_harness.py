@@ -1,0 +1,67 @@
+"""The C++ host harnesses (tests/host): the reference's test/test_correctness.cu and
+test/benchmark.cu flows -- pack() on the host, hipMalloc/hipMemcpy, linear_vN_launch or the
+C ABI, CPU comparison / event timing -- as plain host programs linked against the library."""
+import re
+import subprocess
+from pathlib import Path
+
+import pytest
+
+HOST = Path(__file__).resolve().parent / "host"
+BIN = HOST / "bin"
+
+
+def _binary(name: str) -> Path:
+    exe = BIN / name
+    if not exe.exists():  # built by __graft_entry__.build(); build here only if nothing is there
+        subprocess.run(["make", "-C", str(HOST)], check=True, capture_output=True, text=True)
+    assert exe.exists(), exe
+    return exe
+
+
+def test_harness_binaries_link_against_the_library():
+    for name in ("correctness", "benchmark"):
+        out = subprocess.run(["ldd", str(_binary(name))], check=True, capture_output=True, text=True).stdout
+        assert "libint4linear.so" in out and "not found" not in out, out
+
+
+def test_harness_usage_errors_without_a_device():
+    r = subprocess.run([str(_binary("correctness")), "--entry", "v99", "16x16x128"], capture_output=True, text=True)
+    assert r.returncode == 2
+    r = subprocess.run([str(_binary("benchmark")), "--kernel", "nope"], capture_output=True, text=True)
+    assert r.returncode == 2
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("entry", ["v21", "v20", "v11", "v10", "v2", "v1", "v0", "c"])
+def test_correctness_harness_every_entry_point(gpu, entry):
+    r = subprocess.run([str(_binary("correctness")), "--entry", entry, "--seed", "7",
+                        "300x520x512", "16x1024x1024", "33x70x72"],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert r.stdout.count("TEST PASSED!") == 3 and "FAILED" not in r.stdout
+
+
+@pytest.mark.gpu
+def test_correctness_harness_benchmark_configs(gpu):
+    # cfg1 in full; one large square and one long-K shape on sampled rows; decode shapes with
+    # normal(0, 2) activations.
+    r = subprocess.run([str(_binary("correctness")), "--threads", "16", "1024x1024x1024"],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and "TEST PASSED!" in r.stdout, r.stdout + r.stderr
+    r = subprocess.run([str(_binary("correctness")), "--threads", "16", "--rows", "24", "4096x4096x4096", "2048x2048x4096"],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and r.stdout.count("TEST PASSED!") == 2, r.stdout + r.stderr
+    r = subprocess.run([str(_binary("correctness")), "--threads", "16", "--dist", "normal",
+                        "16x14336x4096", "1x4096x14336", "64x4096x4096"],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and r.stdout.count("TEST PASSED!") == 3, r.stdout + r.stderr
+
+
+@pytest.mark.gpu
+def test_benchmark_harness_reports_tops(gpu):
+    r = subprocess.run([str(_binary("benchmark")), "--iters", "5", "--warmup", "2", "2048x2048x2048", "16x4096x4096"],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout + r.stderr
+    lines = re.findall(r"\[PERF\] (\d+)x(\d+)x(\d+) kernel=(\w+) median ([\d.]+) ms .* ([\d.]+) TOPS", r.stdout)
+    assert len(lines) == 2 and all(float(l[5]) > 0 for l in lines), r.stdout
