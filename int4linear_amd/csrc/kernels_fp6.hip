@@ -11,11 +11,12 @@
 // arithmetic (the tests compare it against the CPU oracle).
 //
 // Two kernels:
-//   * fp6_convert_kernel rewrites a packed s4 operand (rows x K/2 bytes) into FP6
+//   * fp6_convert_kernel rewrites packed s4 operands (rows x K/2 bytes) into FP6
 //     "fragment-major" form in a workspace: for every block of 32 rows x 64 k the 24
 //     bytes each of the 64 MFMA lanes feeds to the instruction, stored as 64 x 16 B
 //     followed by 64 x 8 B.  Rows are padded with zeros to a multiple of the 256-row
-//     tile.  HBM-bound: 0.5 B read and 0.75 B written per element.
+//     tile.  One launch converts both operands.  HBM-bound: 0.5 B read and 0.75 B
+//     written per element.
 //   * fp6_gemm_kernel is a persistent, LDS-pipelined GEMM over those fragments.  Because
 //     the workspace is already in the order lanes consume it, global->LDS is a linear
 //     direct-to-LDS copy, LDS->VGPR is one 16-byte and one 8-byte read per lane per
@@ -92,39 +93,74 @@ __device__ __forceinline__ size_t frag_offset(int tile, int stage, int kf, int r
     return ((((size_t)tile * stages + stage) * kFragsK + kf) * kFragsRows + rf) * (size_t)kFragBytes;
 }
 
-// One workgroup converts 32 rows x 256 k.  Thread t handles row t/8 and the 16-byte chunk
-// t%8 (32 k): eight neighbouring lanes read 128 contiguous bytes of a row and write 128
-// contiguous bytes of a fragment's 16-byte parts.
-__global__ __launch_bounds__(256) void fp6_convert_kernel(const uint8_t *__restrict__ src,
-                                                           uint8_t *__restrict__ ws, int rows,
-                                                           int padded_rows, int k)
+// One operand of a conversion launch.
+struct ConvertJob {
+    const uint8_t *src;   // packed s4, rows x k/2 bytes
+    uint8_t *dst;         // fragment-major FP6
+    int rows;             // real rows; rows up to the next multiple of 256 are written as zeros
+    int row_blocks;       // 32-row blocks including the padding
+};
+
+constexpr int kConvK = 512;                          // k per converter workgroup
+constexpr int kConvFrags = kConvK / kFragK;          // 8 fragments out
+constexpr int kConvChunks = kConvK / 32;             // 16-byte input chunks per row
+
+// One workgroup converts 32 rows x 512 k of one operand: thread t reads the 16-byte chunks
+// t%8 and t%8 + 8 of row t/8 (eight neighbouring lanes fetch a whole 128-byte line), the
+// FP6 fragments are assembled in LDS, and the eight finished fragments (1536 contiguous
+// bytes each) leave with full-line 16-byte stores.  blockIdx.y selects the operand and the
+// 32-row block, so one launch converts both A and B.
+__global__ __launch_bounds__(256) void fp6_convert_kernel(ConvertJob ja, ConvertJob jb, int k)
 {
+    __shared__ __attribute__((aligned(16))) uint8_t out[kConvFrags * kFragBytes];
+    const bool second = (int)blockIdx.y >= ja.row_blocks;
+    const ConvertJob job = second ? jb : ja;
+    const int rb = second ? blockIdx.y - ja.row_blocks : blockIdx.y;
     const int r = threadIdx.x >> 3;
     const int c = threadIdx.x & 7;
-    const int row = blockIdx.y * kFragRows + r;       // < padded_rows
-    const int kchunk = blockIdx.x * 8 + c;            // 32-k chunk index along the row
+    const int row = rb * kFragRows + r;
     const int stages = k / kStageK;
-    if (kchunk * 32 >= k)  // K % 256 == 128: the last workgroup of a row is half empty
-        return;
-    v4i w = {0, 0, 0, 0};
-    if (row < rows)
-        w = __builtin_nontemporal_load((const v4i *)(src + (size_t)row * (k >> 1) + (size_t)kchunk * 16));
-    const unsigned long long q0 = fp6_from_dword((unsigned)w[0]);
-    const unsigned long long q1 = fp6_from_dword((unsigned)w[1]);
-    const unsigned long long q2 = fp6_from_dword((unsigned)w[2]);
-    const unsigned long long q3 = fp6_from_dword((unsigned)w[3]);
-    const unsigned long long o0 = q0 | (q1 << 48);
-    const unsigned long long o1 = (q1 >> 16) | (q2 << 32);
-    const unsigned long long o2 = (q2 >> 32) | (q3 << 16);
+    const int kchunk0 = blockIdx.x * kConvChunks;
+    const int chunks_here = min(kConvChunks, (k >> 5) - kchunk0);   // K % 512 may be 128..384
 
-    const int kfrag = kchunk >> 1;                    // 64-k fragment index along the row
-    const int lane = (kchunk & 1) * 32 + (row & 31);
-    uint8_t *frag = ws + frag_offset(row / kTileRows, kfrag / kFragsK, kfrag % kFragsK,
-                                     (row % kTileRows) / kFragRows, stages);
-    const v4i lo = {(int)o0, (int)(o0 >> 32), (int)o1, (int)(o1 >> 32)};
-    const v2i hi = {(int)o2, (int)(o2 >> 32)};
-    *(v4i *)(frag + lane * 16) = lo;
-    *(v2i *)(frag + kFragLoBytes + lane * 8) = hi;
+    v4i w[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int kc = c + 8 * h;
+        w[h] = (v4i){0, 0, 0, 0};
+        if (row < job.rows && kc < chunks_here)
+            w[h] = __builtin_nontemporal_load(
+                (const v4i *)(job.src + (size_t)row * (k >> 1) + (size_t)(kchunk0 + kc) * 16));
+    }
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const unsigned long long q0 = fp6_from_dword((unsigned)w[h][0]);
+        const unsigned long long q1 = fp6_from_dword((unsigned)w[h][1]);
+        const unsigned long long q2 = fp6_from_dword((unsigned)w[h][2]);
+        const unsigned long long q3 = fp6_from_dword((unsigned)w[h][3]);
+        const unsigned long long o0 = q0 | (q1 << 48);
+        const unsigned long long o1 = (q1 >> 16) | (q2 << 32);
+        const unsigned long long o2 = (q2 >> 32) | (q3 << 16);
+        const int kc = c + 8 * h;
+        const int lane = (kc & 1) * 32 + r;
+        uint8_t *frag = out + (kc >> 1) * kFragBytes;
+        *(v4i *)(frag + lane * 16) = (v4i){(int)o0, (int)(o0 >> 32), (int)o1, (int)(o1 >> 32)};
+        *(v2i *)(frag + kFragLoBytes + lane * 8) = (v2i){(int)o2, (int)(o2 >> 32)};
+    }
+    __syncthreads();
+
+    // Fragment f of this workgroup is k-fragment kfrag0 + f of the row block.
+    const int tile = row / kTileRows;                 // uniform in the workgroup
+    const int rf = rb % kFragsRows;
+    const int kfrag0 = kchunk0 >> 1;
+    const int frags_here = chunks_here >> 1;
+    constexpr int kVecPerFrag = kFragBytes / 16;      // 96
+    for (int i = threadIdx.x; i < frags_here * kVecPerFrag; i += 256) {
+        const int f = i / kVecPerFrag, v = i % kVecPerFrag;
+        const int kfrag = kfrag0 + f;
+        uint8_t *dst = job.dst + frag_offset(tile, kfrag / kFragsK, kfrag % kFragsK, rf, stages);
+        *(v4i *)(dst + v * 16) = *(const v4i *)(out + f * kFragBytes + v * 16);
+    }
 }
 
 // ---- GEMM ---------------------------------------------------------------------------------
@@ -447,16 +483,30 @@ hipError_t fp6_init(const DeviceInfo &dev)
 
 size_t fp6_operand_bytes(int rows, int k) { return operand_ws_bytes(rows, k); }
 
-hipError_t launch_fp6_convert(const void *src, void *dst, int rows, int k, hipStream_t stream)
+namespace {
+
+ConvertJob make_job(const void *src, void *dst, int rows)
 {
     const int tiles = (rows + kTileRows - 1) / kTileRows;
-    if (tiles * kFragsRows > 65535)
+    return ConvertJob{(const uint8_t *)src, (uint8_t *)dst, rows, tiles * kFragsRows};
+}
+
+hipError_t launch_convert_jobs(const ConvertJob &ja, const ConvertJob &jb, int k, hipStream_t stream)
+{
+    const int yblocks = ja.row_blocks + jb.row_blocks;
+    if (yblocks > 65535)
         return hipErrorInvalidValue;
-    // One converter workgroup per 32 rows x 256 k (K % 256 may be 128: the kernel guards).
-    const int kblocks = (k + 255) / 256;
-    fp6_convert_kernel<<<dim3(kblocks, tiles * kFragsRows), 256, 0, stream>>>(
-        (const uint8_t *)src, (uint8_t *)dst, rows, tiles * kTileRows, k);
+    if (yblocks == 0)
+        return hipSuccess;
+    fp6_convert_kernel<<<dim3((k + kConvK - 1) / kConvK, yblocks), 256, 0, stream>>>(ja, jb, k);
     return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_fp6_convert(const void *src, void *dst, int rows, int k, hipStream_t stream)
+{
+    return launch_convert_jobs(make_job(src, dst, rows), ConvertJob{nullptr, nullptr, 0, 0}, k, stream);
 }
 
 hipError_t launch_fp6_gemm(const void *a_conv, const void *b_conv, void *c, int m, int n, int k,
@@ -481,9 +531,7 @@ hipError_t launch_fp6(const void *a, const void *b, void *c, int m, int n, int k
 {
     uint8_t *xws = (uint8_t *)workspace;
     uint8_t *wws = xws + operand_ws_bytes(m, k);
-    hipError_t e = launch_fp6_convert(a, xws, m, k, stream);
-    if (e == hipSuccess)
-        e = launch_fp6_convert(b, wws, n, k, stream);
+    hipError_t e = launch_convert_jobs(make_job(a, xws, m), make_job(b, wws, n), k, stream);
     if (e == hipSuccess)
         e = launch_fp6_gemm(xws, wws, c, m, n, k, dev, stream);
     return e;
