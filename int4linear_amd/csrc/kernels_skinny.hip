@@ -21,6 +21,8 @@
 // No atomics, no workspace, and the result does not depend on timing.
 #include "kernels.h"
 
+#include <utility>
+
 namespace int4linear {
 
 namespace {
@@ -56,13 +58,41 @@ __device__ __forceinline__ void dma16(const void *gptr, unsigned lds_addr)
 // bank groups of the 256-byte bank window.
 __device__ __forceinline__ int slot_swizzle(int r) { return (r >> 1) & 7; }
 
+// Waits until at most n of this wave's vector-memory operations are outstanding
+// (they complete in issue order).  n is a compile-time constant at every call site after
+// unrolling; s_waitcnt needs it as an immediate: vmcnt[3:0] in bits 3:0, vmcnt[5:4] in
+// bits 15:14, the other counters left at "no wait".
+template <int N>
+__device__ __forceinline__ void wait_vm_imm()
+{
+    static_assert(N >= 0 && N <= 63, "vmcnt is six bits");
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 0xF) | (((N >> 4) & 0x3) << 14));
+}
+
+// 16 bytes per lane from global memory into registers, invisible to the compiler's own
+// wait-count bookkeeping (which would otherwise wait for the younger weight loads too).
+// The value is only valid after a wait_vm_imm that covers it and a settle().
+__device__ __forceinline__ void load16_untracked(v4i &dst, const void *gptr)
+{
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(gptr) : "memory");
+}
+__device__ __forceinline__ void settle(v4i &v) { asm volatile("" : "+v"(v)); }
+
 // T tiles per wave, R row groups per workgroup, FMX 16-row groups of X (M <= 16*FMX).
 // XDMA: X tiles go through LDS like W; otherwise they are loaded into registers in
 // fragment layout (for K so long that X tiles do not fit in LDS next to the W staging).
+//
+// A workgroup owns rows [blockIdx.x * rows_blk, + rows_blk) of W, rows_blk a multiple of 8
+// and at most 16*R.  Every wave issues all its loads up front in the order X, then row
+// group 0, 1, ...; since loads complete in order, "row group rg, tile t has landed" is a
+// wait for a fixed number of younger loads.  Each row group is multiplied, reduced across
+// the waves and stored as soon as it has landed, while the later groups are still in
+// flight, so only the last group's reduction is exposed after the last byte arrives.
 template <int T, int R, int FMX, bool XDMA>
 __global__ __launch_bounds__(1024) void skinny_kernel(const uint8_t *__restrict__ X,
                                                       const uint8_t *__restrict__ W,
-                                                      int32_t *__restrict__ Y, int M, int N, int K)
+                                                      int32_t *__restrict__ Y, int M, int N, int K,
+                                                      int rows_blk)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int kWaveTiles = T * (R + (XDMA ? FMX : 0));
@@ -71,125 +101,150 @@ __global__ __launch_bounds__(1024) void skinny_kernel(const uint8_t *__restrict_
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int waves = blockDim.x >> 6;  // S
     const int rowbytes = K >> 1;
-    const int n0 = blockIdx.x * 16 * R;
+    const int n0 = blockIdx.x * rows_blk;
+    const int n_end = min(N, n0 + rows_blk);  // > n0
     const unsigned lds_base = (unsigned)(size_t)I4L_LDS(lds);
     const unsigned my_lds = lds_base + wave * kWaveTiles * kTileBytes;
     const size_t kbyte0 = (size_t)wave * T * kTileRowBytes;  // this wave's slice of every row
 
-    // ---- loads.  Lane p of a load instruction lands in LDS at 16*p: tile row p/8 (+8 for
-    //      the second instruction of a tile), slot p%8, so it fetches chunk slot ^ swizzle.
-    {
-        const int lrow = lane >> 3;
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            const int row = lrow + 8 * u;
-            const int chunk = (lane & 7) ^ slot_swizzle(row);
-#pragma unroll
-            for (int rg = 0; rg < R; ++rg) {
-                const int wr = n0 + rg * 16 + row;
-                const uint8_t *src = W + (size_t)(wr < N ? wr : N - 1) * rowbytes + kbyte0 + chunk * 16;
-#pragma unroll
-                for (int t = 0; t < T; ++t)
-                    dma16<true>(src + t * kTileRowBytes, my_lds + (rg * T + t) * kTileBytes + u * 1024);
-            }
-            if (XDMA) {
-#pragma unroll
-                for (int f = 0; f < FMX; ++f) {
-                    const int xr = f * 16 + row;
-                    const uint8_t *src = X + (size_t)(xr < M ? xr : M - 1) * rowbytes + kbyte0 + chunk * 16;
-#pragma unroll
-                    for (int t = 0; t < T; ++t)
-                        dma16<false>(src + t * kTileRowBytes,
-                                     my_lds + ((R + f) * T + t) * kTileBytes + u * 1024);
-                }
-            }
-        }
-    }
-
-    // ---- fragment layout: lane l supplies row l%16 and, in step s of a tile, chunk
-    //      4*s + l/16 (32 nibbles: even ones feed one MFMA, odd ones the next).
+    // Fragment layout: lane l supplies row l%16 and, in step s of a tile, chunk
+    // 4*s + l/16 (32 nibbles: even ones feed one MFMA, odd ones the next).
     const int fr = lane & 15;
     const int fg = lane >> 4;
     const int sw = slot_swizzle(fr);
+
+    // ---- loads.  Lane p of a direct-to-LDS instruction lands at 16*p: tile row p/8 (+8
+    //      for the second instruction of a tile), slot p%8, so it fetches chunk
+    //      slot ^ swizzle.  Rows past the workgroup's (or the matrix's) end re-read the
+    //      last valid row: every wave issues the same number of loads, which the waits
+    //      below rely on, and nothing is read out of bounds.
     v4i xg[XDMA ? 1 : T][2][FMX];
-    if (!XDMA) {
+    {
+        const int lrow = lane >> 3;
+        int chunk[2];
 #pragma unroll
-        for (int f = 0; f < FMX; ++f) {
-            const int xr = f * 16 + fr;
-            const uint8_t *src = X + (size_t)(xr < M ? xr : M - 1) * rowbytes + kbyte0;
+        for (int u = 0; u < 2; ++u)
+            chunk[u] = ((lane & 7) ^ slot_swizzle(lrow + 8 * u)) * 16;
+        if (XDMA) {
+#pragma unroll
+            for (int f = 0; f < FMX; ++f)
+#pragma unroll
+                for (int t = 0; t < T; ++t)
+#pragma unroll
+                    for (int u = 0; u < 2; ++u) {
+                        const int xr = f * 16 + lrow + 8 * u;
+                        const uint8_t *src = X + (size_t)(xr < M ? xr : M - 1) * rowbytes + kbyte0 + chunk[u];
+                        dma16<false>(src + t * kTileRowBytes,
+                                     my_lds + ((R + f) * T + t) * kTileBytes + u * 1024);
+                    }
+        } else {
+#pragma unroll
+            for (int f = 0; f < FMX; ++f) {
+                const int xr = f * 16 + fr;
+                const uint8_t *src = X + (size_t)(xr < M ? xr : M - 1) * rowbytes + kbyte0;
+#pragma unroll
+                for (int t = 0; t < T; ++t)
+#pragma unroll
+                    for (int s = 0; s < 2; ++s)
+                        load16_untracked(xg[t][s][f], src + t * kTileRowBytes + (4 * s + fg) * 16);
+            }
+        }
+#pragma unroll
+        for (int rg = 0; rg < R; ++rg)
 #pragma unroll
             for (int t = 0; t < T; ++t)
 #pragma unroll
-                for (int s = 0; s < 2; ++s)
-                    xg[t][s][f] = *(const v4i *)(src + t * kTileRowBytes + (4 * s + fg) * 16);
-        }
-    }
-
-    v4i acc[R][FMX];
-#pragma unroll
-    for (int rg = 0; rg < R; ++rg)
-#pragma unroll
-        for (int f = 0; f < FMX; ++f)
-            acc[rg][f] = (v4i){0, 0, 0, 0};
-    const int himask = (int)0xF0F0F0F0u;
-
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    const uint8_t *mine = lds + wave * kWaveTiles * kTileBytes;
-#pragma unroll
-    for (int t = 0; t < T; ++t) {
-#pragma unroll
-        for (int s = 0; s < 2; ++s) {
-            const int off = fr * kTileRowBytes + (((4 * s + fg) ^ sw) * 16);
-            v4i xlo[FMX], xhi[FMX];
-#pragma unroll
-            for (int f = 0; f < FMX; ++f) {
-                const v4i x = XDMA ? *(const v4i *)(mine + ((R + f) * T + t) * kTileBytes + off) : xg[XDMA ? 0 : t][s][f];
-                xlo[f] = (x << 4) & himask;
-                xhi[f] = x & himask;
-            }
-#pragma unroll
-            for (int rg = 0; rg < R; ++rg) {
-                const v4i w = *(const v4i *)(mine + (rg * T + t) * kTileBytes + off);
-                const v4i wlo = (w << 4) & himask;
-                const v4i whi = w & himask;
-#pragma unroll
-                for (int f = 0; f < FMX; ++f) {
-                    acc[rg][f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo, xlo[f], acc[rg][f], 0, 0, 0);
-                    acc[rg][f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi, xhi[f], acc[rg][f], 0, 0, 0);
+                for (int u = 0; u < 2; ++u) {
+                    const int wr = n0 + rg * 16 + lrow + 8 * u;
+                    const uint8_t *src = W + (size_t)(wr < n_end ? wr : n_end - 1) * rowbytes + kbyte0 + chunk[u];
+                    dma16<true>(src + t * kTileRowBytes, my_lds + (rg * T + t) * kTileBytes + u * 1024);
                 }
-            }
-        }
     }
 
-    // ---- the S partial sums of every output meet in LDS (the staging area is free now)
-    __syncthreads();
-    v4i *partial = (v4i *)lds;  // [R*FMX][waves][64]
-#pragma unroll
-    for (int rg = 0; rg < R; ++rg)
-#pragma unroll
-        for (int f = 0; f < FMX; ++f)
-            partial[((rg * FMX + f) * waves + wave) * 64 + lane] = acc[rg][f];
-    __syncthreads();
+    const int himask = (int)0xF0F0F0F0u;
+    const uint8_t *mine = lds + wave * kWaveTiles * kTileBytes;
 
-    // Element e = (rg, f, lane): n = n0 + 16*rg + 4*(lane/16) + 0..3, m = 16*f + lane%16.
-    for (int e = threadIdx.x; e < R * FMX * 64; e += blockDim.x) {
-        const int q = e >> 6, l = e & 63;
-        const v4i *p = partial + (size_t)q * waves * 64 + l;
-        v4i s = p[0];
-        for (int wv = 1; wv < waves; ++wv)
-            s += p[wv * 64];
-        s = s >> 8;  // both operands carried a factor 16
-        const int m = (q % FMX) * 16 + (l & 15);
-        const int n = n0 + (q / FMX) * 16 + 4 * (l >> 4);
+    // ---- one row group at a time
+    [&]<int... RG>(std::integer_sequence<int, RG...>) {
+        ([&] {
+            constexpr int rg = RG;
+            v4i acc[FMX];
+#pragma unroll
+            for (int f = 0; f < FMX; ++f)
+                acc[f] = (v4i){0, 0, 0, 0};
+            [&]<int... TT>(std::integer_sequence<int, TT...>) {
+                ([&] {
+                    constexpr int t = TT;
+                    // loads younger than tile (rg, t): the rest of this group and the later groups
+                    wait_vm_imm<((R - 1 - rg) * T + (T - 1 - t)) * 2>();
+                    if (!XDMA && rg == 0 && t == 0) {
+#pragma unroll
+                        for (int tt = 0; tt < (XDMA ? 1 : T); ++tt)
+#pragma unroll
+                            for (int s = 0; s < 2; ++s)
+#pragma unroll
+                                for (int f = 0; f < FMX; ++f)
+                                    settle(xg[tt][s][f]);
+                    }
+#pragma unroll
+                    for (int s = 0; s < 2; ++s) {
+                        const int off = fr * kTileRowBytes + (((4 * s + fg) ^ sw) * 16);
+                        const v4i w = *(const v4i *)(mine + (rg * T + t) * kTileBytes + off);
+                        const v4i wlo = (w << 4) & himask;
+                        const v4i whi = w & himask;
+#pragma unroll
+                        for (int f = 0; f < FMX; ++f) {
+                            const v4i x = XDMA ? *(const v4i *)(mine + ((R + f) * T + t) * kTileBytes + off)
+                                               : xg[XDMA ? 0 : t][s][f];
+                            acc[f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo, (x << 4) & himask, acc[f], 0, 0, 0);
+                            acc[f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi, x & himask, acc[f], 0, 0, 0);
+                        }
+                    }
+                }(), ...);
+            }(std::make_integer_sequence<int, T>{});
+
+            // The wave's partial sums of this group go where its own tiles of the group
+            // were (nobody else touches that area).
+            v4i *part = (v4i *)(mine + (rg * T) * kTileBytes);
+#pragma unroll
+            for (int f = 0; f < FMX; ++f)
+                part[f * 64 + lane] = acc[f];
+        }(), ...);
+    }(std::make_integer_sequence<int, R>{});
+
+    // ---- the workgroup meets once; one wave per 16 x 16 block adds the S partials up
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's partials are in LDS
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int b = 0; b < R * FMX; ++b) {
+        if (wave != b % waves)
+            continue;
+        const int rg = b / FMX, f = b % FMX;
+        const v4i *p = (const v4i *)(lds + (rg * T) * kTileBytes) + f * 64 + lane;
+        // All sixteen reads are issued back to back (a loop over the runtime wave count
+        // would wait for each one); waves that do not exist re-read partial 0 and add zero.
+        v4i part[16];
+#pragma unroll
+        for (int wv = 0; wv < 16; ++wv)
+            part[wv] = p[(size_t)(wv < waves ? wv : 0) * (kWaveTiles * kTileBytes / 16)];
+        v4i sum = part[0];
+#pragma unroll
+        for (int wv = 1; wv < 16; ++wv)
+            sum += wv < waves ? part[wv] : (v4i){0, 0, 0, 0};
+        sum = sum >> 8;  // both operands carried a factor 16
+        // lane l: m = 16*f + l%16, n = n0 + 16*rg + 4*(l/16) + 0..3
+        const int m = f * 16 + fr;
+        const int n = n0 + rg * 16 + 4 * fg;
         if (m < M) {
             int32_t *dst = Y + (size_t)m * N + n;
-            if (n + 3 < N && (N & 3) == 0) {
-                *(v4i *)dst = s;
+            if (n + 3 < n_end && (N & 3) == 0) {
+                *(v4i *)dst = sum;
             } else {
 #pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    if (n + t < N)
-                        dst[t] = s[t];
+                for (int q = 0; q < 4; ++q)
+                    if (n + q < n_end)
+                        dst[q] = sum[q];
             }
         }
     }
@@ -279,12 +334,14 @@ hipError_t launch_basic(const void *a, const void *b, void *c, int m, int n, int
 
 struct Plan {
     int t = 0, s = 0, r = 0, fmx = 0;
+    int rows_blk = 0;  // rows of W per workgroup: a multiple of 8, <= 16 * r
     bool xdma = true;
     int lds = 0;
 };
 
-// Largest S <= 16 with S * T == tiles for the smallest T <= 4; R as large as keeps
-// R * FMX <= 4, the grid near the CU count and the staging inside LDS.
+// Largest S <= 16 with S * T == tiles for the smallest T <= 4.  Rows per workgroup: the
+// matrix split evenly over the CUs (in as few rounds as the LDS and accumulator limits
+// allow), rounded up to a multiple of 8; R is the number of 16-row groups that takes.
 bool make_plan(int m, int n, int k, int cu_count, Plan &p)
 {
     if (k % kTileK != 0)
@@ -300,29 +357,39 @@ bool make_plan(int m, int n, int k, int cu_count, Plan &p)
         }
     if (p.t == 0)
         return false;
-    auto lds_for = [&](int r, bool xdma) {
-        const int staging = p.s * p.t * (r + (xdma ? p.fmx : 0)) * kTileBytes;
-        const int reduce = r * p.fmx * p.s * 1024;
-        return staging > reduce ? staging : reduce;
-    };
-    for (int r = 4; r >= 1; r >>= 1) {
+    auto lds_for = [&](int r, bool xdma) { return p.s * p.t * (r + (xdma ? p.fmx : 0)) * kTileBytes; };
+    // largest R the limits allow (R in {1, 2, 4}, R * FMX <= 4 accumulator blocks)
+    int rmax = 0;
+    bool xdma = true;
+    for (int r = 4; r >= 1 && rmax == 0; r >>= 1) {
         if (r * p.fmx > 4)
             continue;
-        const long blocks = (n + 16 * r - 1) / (16 * r);
-        if (r > 1 && blocks * 10 < (long)cu_count * 8)
-            continue;  // too few workgroups: prefer smaller R
         for (int xd = 1; xd >= 0; --xd) {
             if (xd == 0 && (p.t != 4 || p.fmx > 2))
                 continue;  // the register-X variant exists for T == 4, M <= 32 only
             if (lds_for(r, xd != 0) <= kMaxLds) {
-                p.r = r;
-                p.xdma = xd != 0;
-                p.lds = lds_for(r, p.xdma);
-                return true;
+                rmax = r;
+                xdma = xd != 0;
+                break;
             }
         }
     }
-    return false;
+    if (rmax == 0)
+        return false;
+    const long cus = cu_count > 0 ? cu_count : 1;
+    const long rounds = (n + cus * 16 * rmax - 1) / (cus * 16 * rmax);
+    const long per_block = (n + cus * rounds - 1) / (cus * rounds);
+    p.rows_blk = (int)((per_block + 7) / 8 * 8);
+    int r = 1;
+    while (16 * r < p.rows_blk)
+        r <<= 1;
+    p.r = r;  // <= rmax
+    // X through LDS whenever it fits for this R
+    p.xdma = lds_for(r, true) <= kMaxLds ? true : xdma;
+    if (!p.xdma && (p.t != 4 || p.fmx > 2))
+        return false;
+    p.lds = lds_for(r, p.xdma);
+    return p.lds <= kMaxLds;
 }
 
 template <int T, int R, int FMX, bool XDMA>
@@ -335,8 +402,9 @@ hipError_t launch_plan(const Plan &p, const void *a, const void *b, void *c, int
     auto kern = skinny_kernel<T, R, FMX, XDMA>;
     if (p.s == 0)  // set-up call: raise the dynamic-LDS limit of this instantiation
         return hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
-    const unsigned grid = (unsigned)((n + 16 * R - 1) / (16 * R));
-    kern<<<grid, p.s * 64, p.lds, stream>>>((const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k);
+    const unsigned grid = (unsigned)((n + p.rows_blk - 1) / p.rows_blk);
+    kern<<<grid, p.s * 64, p.lds, stream>>>((const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k,
+                                            p.rows_blk);
     return hipGetLastError();
     }
 }
