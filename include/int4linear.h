@@ -45,9 +45,11 @@ enum {
     INT4LINEAR_KERNEL_SIMPLE = 1, /* one thread per output, scalar nibble decode; any K%8==0 */
     INT4LINEAR_KERNEL_MFMA = 2,   /* LDS-pipelined v_mfma_i32_32x32x32_i8 kernel; K%128==0 */
     INT4LINEAR_KERNEL_SKINNY = 3, /* weight-streaming kernel for M <= 64; K%128==0       */
-    INT4LINEAR_KERNEL_FP6 = 4     /* operands converted to FP6 (E2M3) in a workspace, then
-                                     v_mfma_scale_f32_32x32x64_f8f6f4; exact; K%128==0,
-                                     K < 2^18                                            */
+    INT4LINEAR_KERNEL_FP6 = 4,    /* operands converted to FP6 (E2M3) in a workspace, then
+                                     v_mfma_scale_f32_32x32x64_f8f6f4; exact; any K%8==0
+                                     below 2^18 (the converter pads K to 128 with zeros) */
+    INT4LINEAR_KERNEL_MFMA_128 = 5, /* the int8 kernel with its 128x128 workgroup tile   */
+    INT4LINEAR_KERNEL_MFMA_256 = 6  /* the int8 kernel with its 256x256 workgroup tile   */
 };
 
 /* One-time set-up for the current HIP device (queries the CU count, raises the
@@ -120,8 +122,17 @@ int int4linear_device_cu_count(void);
 /*
  * The reference's entry points, C++ linkage, same signatures and semantics:
  * blocking (the call returns after the device has finished), default stream, void
- * return, silent on success.  All seven names run the same dispatch; v0 always takes
- * the simple kernel so it can serve as an independent on-device cross-check.
+ * return, silent on success.  As in the reference, each name is one step of the
+ * optimisation history, here the one of this library's kernels:
+ *   v0   scalar kernel, no matrix cores (also the independent on-device cross-check)
+ *   v1   int8 MFMA kernel, 128x128 workgroup tile
+ *   v2   int8 MFMA kernel, 256x256 workgroup tile
+ *   v10  int8 MFMA kernel, tile chosen from the grid size
+ *   v11  v10 plus the weight-streaming kernel for M <= 64
+ *   v20  v11 plus the FP6 kernel wherever it can run
+ *   v21  the full automatic dispatch (what int4linear_gemm_s4s4s32 does)
+ * A version whose kernel cannot take a shape falls back to the one before it, so every
+ * name accepts every valid shape.
  *   kernels/linear_v0.h:168   kernels/linear_v1.h:208   kernels/linear_v2.h:284
  *   kernels/linear_v10.h:492  kernels/linear_v11.h:658  kernels/linear_v20.h:738
  *   kernels/linear_v21.h:760

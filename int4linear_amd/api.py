@@ -14,7 +14,7 @@ import numpy as np
 
 from . import _lib
 
-KERNELS = {"auto": 0, "simple": 1, "mfma": 2, "skinny": 3, "fp6": 4}
+KERNELS = {"auto": 0, "simple": 1, "mfma": 2, "skinny": 3, "fp6": 4, "mfma128": 5, "mfma256": 6}
 
 
 def _ptr(obj) -> int:

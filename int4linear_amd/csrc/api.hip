@@ -92,6 +92,15 @@ bool fp6_worthwhile(int m, int n, int k)
            fp6_workspace_bytes(m, n, k) <= g_workspace_limit.load();
 }
 
+// K that is not a multiple of 128 fits neither the int8 nor the weight-streaming kernel,
+// but the FP6 converter pads K with zeros: beyond a few million multiply-adds that beats
+// the scalar kernel by orders of magnitude even for a handful of rows.
+bool fp6_for_ragged_k(int m, int n, int k)
+{
+    return (k % 128) != 0 && fp6_supports(m, n, k) && (double)m * n * k >= (double)(1 << 22) &&
+           fp6_workspace_bytes(m, n, k) <= g_workspace_limit.load();
+}
+
 int pick_kernel(int m, int n, int k)
 {
     if (skinny_supports(m, n, k))
@@ -100,6 +109,8 @@ int pick_kernel(int m, int n, int k)
         return INT4LINEAR_KERNEL_FP6;
     if (mfma_supports(m, n, k))
         return INT4LINEAR_KERNEL_MFMA;
+    if (fp6_for_ragged_k(m, n, k))
+        return INT4LINEAR_KERNEL_FP6;
     return INT4LINEAR_KERNEL_SIMPLE;
 }
 
@@ -156,7 +167,7 @@ int gemm_impl(const void *a, const void *b, void *c, int m, int n, int k, int ke
 {
     if (m < 0 || n < 0 || k < 0 || (k % 8) != 0)
         return INT4LINEAR_ERR_SHAPE;
-    if (kernel < INT4LINEAR_KERNEL_AUTO || kernel > INT4LINEAR_KERNEL_FP6)
+    if (kernel < INT4LINEAR_KERNEL_AUTO || kernel > INT4LINEAR_KERNEL_MFMA_256)
         return INT4LINEAR_ERR_UNSUPPORTED;
     if (m == 0 || n == 0)
         return INT4LINEAR_OK;
@@ -185,11 +196,11 @@ int gemm_impl(const void *a, const void *b, void *c, int m, int n, int k, int ke
         if (!fp6_supports(m, n, k))
             return INT4LINEAR_ERR_UNSUPPORTED;
         const int st6 = run_fp6(pd, a, b, c, m, n, k, stream);
-        // Under automatic dispatch a workspace that cannot be had falls back to the
-        // int8 kernel, which needs none.
+        // Under automatic dispatch a workspace that cannot be had falls back to a kernel
+        // that needs none.
         if (st6 == INT4LINEAR_OK || !automatic)
             return st6;
-        kernel = INT4LINEAR_KERNEL_MFMA;
+        kernel = mfma_supports(m, n, k) ? INT4LINEAR_KERNEL_MFMA : INT4LINEAR_KERNEL_SIMPLE;
     }
 
     hipError_t e = hipSuccess;
@@ -201,6 +212,13 @@ int gemm_impl(const void *a, const void *b, void *c, int m, int n, int k, int ke
         if (!mfma_supports(m, n, k))
             return INT4LINEAR_ERR_UNSUPPORTED;
         e = launch_mfma(a, b, c, m, n, k, pd->info, stream);
+        break;
+    case INT4LINEAR_KERNEL_MFMA_128:
+    case INT4LINEAR_KERNEL_MFMA_256:
+        if (!mfma_supports(m, n, k))
+            return INT4LINEAR_ERR_UNSUPPORTED;
+        e = launch_mfma_tile(a, b, c, m, n, k, kernel == INT4LINEAR_KERNEL_MFMA_128 ? 128 : 256, pd->info,
+                             stream);
         break;
     case INT4LINEAR_KERNEL_SKINNY:
         if (!skinny_supports(m, n, k))
@@ -402,31 +420,69 @@ int int4linear_device_cu_count(void)
 
 // ---- the reference's C++-linkage entry points ------------------------------------------
 
+namespace {
+
+// Kernel of each step of the version history for a shape; a step whose kernel cannot take
+// the shape falls back to the step before it.
+int version_kernel(int version, int m, int n, int k)
+{
+    const bool int8_ok = mfma_supports(m, n, k);
+    switch (version) {
+    case 21:
+        return INT4LINEAR_KERNEL_AUTO;
+    case 20:
+        if (fp6_supports(m, n, k) && fp6_workspace_bytes(m, n, k) <= g_workspace_limit.load() &&
+            !skinny_supports(m, n, k))
+            return INT4LINEAR_KERNEL_FP6;
+        [[fallthrough]];
+    case 11:
+        if (skinny_supports(m, n, k))
+            return INT4LINEAR_KERNEL_SKINNY;
+        [[fallthrough]];
+    case 10:
+        return int8_ok ? INT4LINEAR_KERNEL_MFMA : INT4LINEAR_KERNEL_SIMPLE;
+    case 2:
+        return int8_ok ? INT4LINEAR_KERNEL_MFMA_256 : INT4LINEAR_KERNEL_SIMPLE;
+    case 1:
+        return int8_ok ? INT4LINEAR_KERNEL_MFMA_128 : INT4LINEAR_KERNEL_SIMPLE;
+    default:
+        return INT4LINEAR_KERNEL_SIMPLE;
+    }
+}
+
+void launch_version(const char *name, int version, void *x, void *w, void *y, int m, int n, int k)
+{
+    const bool valid = m >= 0 && n >= 0 && k >= 0 && (k % 8) == 0;
+    launch_blocking(name, x, w, y, m, n, k, valid ? version_kernel(version, m, n, k) : INT4LINEAR_KERNEL_AUTO);
+}
+
+}  // namespace
+
 void linear_v0_launch(void *x, void *w, void *y, int m, int n, int k)
 {
-    launch_blocking("linear_v0_launch", x, w, y, m, n, k, INT4LINEAR_KERNEL_SIMPLE);
+    launch_version("linear_v0_launch", 0, x, w, y, m, n, k);
 }
 void linear_v1_launch(void *x, void *w, void *y, int m, int n, int k)
 {
-    launch_blocking("linear_v1_launch", x, w, y, m, n, k, INT4LINEAR_KERNEL_AUTO);
+    launch_version("linear_v1_launch", 1, x, w, y, m, n, k);
 }
 void linear_v2_launch(void *x, void *w, void *y, int m, int n, int k)
 {
-    launch_blocking("linear_v2_launch", x, w, y, m, n, k, INT4LINEAR_KERNEL_AUTO);
+    launch_version("linear_v2_launch", 2, x, w, y, m, n, k);
 }
 void linear_v10_launch(void *x, void *w, void *y, int m, int n, int k)
 {
-    launch_blocking("linear_v10_launch", x, w, y, m, n, k, INT4LINEAR_KERNEL_AUTO);
+    launch_version("linear_v10_launch", 10, x, w, y, m, n, k);
 }
 void linear_v11_launch(void *x, void *w, void *y, int m, int n, int k)
 {
-    launch_blocking("linear_v11_launch", x, w, y, m, n, k, INT4LINEAR_KERNEL_AUTO);
+    launch_version("linear_v11_launch", 11, x, w, y, m, n, k);
 }
 void linear_v20_launch(void *x, void *w, void *y, int m, int n, int k)
 {
-    launch_blocking("linear_v20_launch", x, w, y, m, n, k, INT4LINEAR_KERNEL_AUTO);
+    launch_version("linear_v20_launch", 20, x, w, y, m, n, k);
 }
 void linear_v21_launch(void *x, void *w, void *y, int m, int n, int k)
 {
-    launch_blocking("linear_v21_launch", x, w, y, m, n, k, INT4LINEAR_KERNEL_AUTO);
+    launch_version("linear_v21_launch", 21, x, w, y, m, n, k);
 }

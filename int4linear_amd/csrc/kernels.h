@@ -21,6 +21,10 @@ hipError_t mfma_init(const DeviceInfo &dev);
 hipError_t launch_mfma(const void *a, const void *b, void *c, int m, int n, int k,
                        const DeviceInfo &dev, hipStream_t stream);
 
+// The same kernel with the workgroup tile forced to 128 x 128 or 256 x 256 (`tile`).
+hipError_t launch_mfma_tile(const void *a, const void *b, void *c, int m, int n, int k, int tile,
+                            const DeviceInfo &dev, hipStream_t stream);
+
 // FP6-MFMA path: converts both operands into a workspace of fp6_workspace_bytes() bytes
 // (256-byte aligned), then runs the GEMM on it.  Requires K % 128 == 0, K < 2^18.
 bool fp6_supports(int m, int n, int k);

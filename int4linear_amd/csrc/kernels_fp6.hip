@@ -110,7 +110,11 @@ constexpr int kConvChunks = kConvK / 32;             // 16-byte input chunks per
 // FP6 fragments are assembled in LDS, and the eight finished fragments (1536 contiguous
 // bytes each) leave with full-line 16-byte stores.  blockIdx.y selects the operand and the
 // 32-row block, so one launch converts both A and B.
-__global__ __launch_bounds__(256) void fp6_convert_kernel(ConvertJob ja, ConvertJob jb, int k)
+// k is the operand's real K (a multiple of 8; the row stride is k/2 bytes), k_pad the next
+// multiple of 128: k positions from k up to k_pad are written as zeros.  ALIGNED16: k is a
+// multiple of 32, so every 16-byte chunk of a row is aligned and entirely inside the row.
+template <bool ALIGNED16>
+__global__ __launch_bounds__(256) void fp6_convert_kernel(ConvertJob ja, ConvertJob jb, int k, int k_pad)
 {
     __shared__ __attribute__((aligned(16))) uint8_t out[kConvFrags * kFragBytes];
     const bool second = (int)blockIdx.y >= ja.row_blocks;
@@ -119,18 +123,26 @@ __global__ __launch_bounds__(256) void fp6_convert_kernel(ConvertJob ja, Convert
     const int r = threadIdx.x >> 3;
     const int c = threadIdx.x & 7;
     const int row = rb * kFragRows + r;
-    const int stages = k / kStageK;
+    const int stages = k_pad / kStageK;
     const int kchunk0 = blockIdx.x * kConvChunks;
-    const int chunks_here = min(kConvChunks, (k >> 5) - kchunk0);   // K % 512 may be 128..384
+    const int chunks_here = min(kConvChunks, (k_pad >> 5) - kchunk0);   // k_pad % 512 may be 128..384
 
     v4i w[2];
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
         const int kc = c + 8 * h;
         w[h] = (v4i){0, 0, 0, 0};
-        if (row < job.rows && kc < chunks_here)
-            w[h] = __builtin_nontemporal_load(
-                (const v4i *)(job.src + (size_t)row * (k >> 1) + (size_t)(kchunk0 + kc) * 16));
+        const int k0 = (kchunk0 + kc) * 32;  // first k of the chunk
+        const uint8_t *src = job.src + (size_t)row * (k >> 1) + (size_t)(kchunk0 + kc) * 16;
+        if (ALIGNED16) {
+            if (row < job.rows && k0 < k)
+                w[h] = __builtin_nontemporal_load((const v4i *)src);
+        } else {
+#pragma unroll
+            for (int d = 0; d < 4; ++d)
+                if (row < job.rows && k0 + 8 * d < k)
+                    w[h][d] = *(const int *)(src + 4 * d);
+        }
     }
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
@@ -457,15 +469,16 @@ using Fp6Cfg = Fp6Config<2, 4, 1>;
 size_t operand_ws_bytes(int rows, int k)
 {
     const size_t tiles = (size_t)(rows + kTileRows - 1) / kTileRows;
-    return tiles * (size_t)(k / kStageK) * (size_t)kOperandStageBytes;
+    return tiles * (size_t)((k + kStageK - 1) / kStageK) * (size_t)kOperandStageBytes;
 }
 
 }  // namespace
 
 bool fp6_supports(int m, int n, int k)
 {
-    // fp32 accumulation of products bounded by 64 stays exact while K * 64 < 2^24.
-    return m >= 1 && n >= 1 && k >= kStageK && k % kStageK == 0 && k < (1 << 18);
+    // fp32 accumulation of products bounded by 64 stays exact while K * 64 < 2^24.  The
+    // converter pads K to a multiple of 128 with zeros, so any K % 8 == 0 is fine.
+    return m >= 1 && n >= 1 && k >= 8 && k % 8 == 0 && k <= (1 << 18) - kStageK;
 }
 
 size_t fp6_workspace_bytes(int m, int n, int k)
@@ -491,6 +504,8 @@ ConvertJob make_job(const void *src, void *dst, int rows)
     return ConvertJob{(const uint8_t *)src, (uint8_t *)dst, rows, tiles * kFragsRows};
 }
 
+int padded_k(int k) { return (k + kStageK - 1) / kStageK * kStageK; }
+
 hipError_t launch_convert_jobs(const ConvertJob &ja, const ConvertJob &jb, int k, hipStream_t stream)
 {
     const int yblocks = ja.row_blocks + jb.row_blocks;
@@ -498,7 +513,12 @@ hipError_t launch_convert_jobs(const ConvertJob &ja, const ConvertJob &jb, int k
         return hipErrorInvalidValue;
     if (yblocks == 0)
         return hipSuccess;
-    fp6_convert_kernel<<<dim3((k + kConvK - 1) / kConvK, yblocks), 256, 0, stream>>>(ja, jb, k);
+    const int k_pad = padded_k(k);
+    const dim3 grid((k_pad + kConvK - 1) / kConvK, yblocks);
+    if (k % 32 == 0)
+        fp6_convert_kernel<true><<<grid, 256, 0, stream>>>(ja, jb, k, k_pad);
+    else
+        fp6_convert_kernel<false><<<grid, 256, 0, stream>>>(ja, jb, k, k_pad);
     return hipGetLastError();
 }
 
@@ -522,7 +542,7 @@ hipError_t launch_fp6_gemm(const void *a_conv, const void *b_conv, void *c, int 
     if (grid > total)
         grid = total;
     fp6_gemm_kernel<C><<<(unsigned)grid, C::THREADS, kLdsBytes, stream>>>(
-        (const uint8_t *)a_conv, (const uint8_t *)b_conv, (int32_t *)c, m, n, k, tiles_m, tiles_n);
+        (const uint8_t *)a_conv, (const uint8_t *)b_conv, (int32_t *)c, m, n, padded_k(k), tiles_m, tiles_n);
     return hipGetLastError();
 }
 

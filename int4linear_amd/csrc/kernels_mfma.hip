@@ -548,6 +548,16 @@ hipError_t mfma_init(const DeviceInfo &dev)
     return set_lds_limit<CfgMedium>();
 }
 
+hipError_t launch_mfma_tile(const void *a, const void *b, void *c, int m, int n, int k, int tile,
+                            const DeviceInfo &dev, hipStream_t stream)
+{
+    if (tile == 256)
+        return launch_cfg<CfgLarge>(a, b, c, m, n, k, dev, stream);
+    if (tile == 128)
+        return launch_cfg<CfgMedium>(a, b, c, m, n, k, dev, stream);
+    return hipErrorInvalidValue;
+}
+
 hipError_t launch_mfma(const void *a, const void *b, void *c, int m, int n, int k,
                        const DeviceInfo &dev, hipStream_t stream)
 {

@@ -2,7 +2,7 @@
 // launches, 50 timed ones, every timed launch preceded by a cache-cleaning fill and bracketed
 // by its own event pair, median reported as 2*M*N*K / t in TOPS ("[PERF] ... TOPS").
 //
-//   benchmark [--kernel auto|simple|mfma|skinny|fp6] [--iters I] [--warmup W] [--no-flush] MxNxK ...
+//   benchmark [--kernel auto|simple|mfma|mfma128|mfma256|skinny|fp6] [--iters I] [--warmup W] [--no-flush] MxNxK ...
 //
 // The reference cleans twice its L2 (benchmark.cu:77-91); an MI355X also has a 256 MiB
 // memory-side cache behind the eight L2s, so the fill here is 512 MiB.  Operand values are
@@ -21,6 +21,8 @@ int kernel_id(const std::string &name)
     if (name == "mfma") return INT4LINEAR_KERNEL_MFMA;
     if (name == "skinny") return INT4LINEAR_KERNEL_SKINNY;
     if (name == "fp6") return INT4LINEAR_KERNEL_FP6;
+    if (name == "mfma128") return INT4LINEAR_KERNEL_MFMA_128;
+    if (name == "mfma256") return INT4LINEAR_KERNEL_MFMA_256;
     return -1;
 }
 
@@ -41,7 +43,7 @@ int main(int argc, char **argv)
         else if (a == "--no-flush") flush = false;
         else if (parse_shape(argv[i], s)) shapes.push_back(s);
         else {
-            std::fprintf(stderr, "usage: %s [--kernel auto|simple|mfma|skinny|fp6] [--iters I] [--warmup W] "
+            std::fprintf(stderr, "usage: %s [--kernel auto|simple|mfma|mfma128|mfma256|skinny|fp6] [--iters I] [--warmup W] "
                                  "[--no-flush] MxNxK ...\n", argv[0]);
             return 2;
         }

@@ -15,9 +15,10 @@ GOLDEN = np.load(helpers.__file__.replace("helpers.py", "golden/int4_gemm_golden
 
 def kernels_for(m, n, k):
     ks = ["auto", "simple"]
+    if k >= 8:
+        ks.append("fp6")  # any K % 8 == 0: the converter pads K
     if k >= 128 and k % 128 == 0:
-        ks.append("mfma")
-        ks.append("fp6")
+        ks += ["mfma", "mfma128", "mfma256"]
         if m <= 64:
             ks.append("skinny")
     return ks
@@ -138,6 +139,23 @@ def test_fp6_converted_operands(gpu, host_threads, m, n, k):
         y.fill_(-1)
 
 
+@pytest.mark.parametrize("m, n, k", [(1000, 3000, 4104), (16, 4096, 4104), (300, 300, 1000), (257, 513, 40),
+                                     (64, 2048, 2040), (512, 512, 136)])
+def test_ragged_k_runs_on_the_fp6_kernel(gpu, host_threads, m, n, k):
+    """K % 128 != 0 (K % 8 == 0): automatic dispatch pads K in the FP6 converter instead of
+    falling back to the scalar kernel."""
+    import int4linear_amd as lib
+
+    x = helpers.uniform_s4(1000 + m, m, k)
+    w = helpers.uniform_s4(1100 + n, n, k)
+    want = oracle.linear_ref(x, w, threads=host_threads)
+    xp, wp = helpers.pack_bytes(x), helpers.pack_bytes(w)
+    assert lib.kernel_for_shape(m, n, k) == "fp6"
+    for kern in ("auto", "fp6"):
+        got = helpers.run_gemm(xp, wp, m, n, k, kernel=kern)
+        assert np.array_equal(got, want), kern
+
+
 # ---- configuration 5: adversarial ---------------------------------------------------------
 
 def test_cfg5_all_minus_eight_full_size(gpu):
@@ -241,6 +259,26 @@ def test_properties_at_4096(gpu):
 
 
 # ---- the reference's blocking entry points ------------------------------------------------------
+
+@pytest.mark.parametrize("shape", [(300, 520, 512), (16, 1024, 1024), (33, 70, 72), (2048, 2304, 256)])
+@pytest.mark.parametrize("version", [0, 1, 2, 10, 11, 20, 21])
+def test_every_version_takes_every_shape(gpu, version, shape):
+    """v0..v21 are different kernels (scalar, int8 128/256 tile, +skinny, +fp6, automatic);
+    a version whose kernel cannot run a shape falls back, so all of them agree everywhere."""
+    import torch
+
+    import int4linear_amd as lib
+
+    m, n, k = shape
+    x = helpers.uniform_s4(900 + version, m, k)
+    w = helpers.uniform_s4(901 + version, n, k)
+    want = oracle.linear_ref(x, w, threads=4)
+    xd = helpers.to_device_bytes(helpers.pack_words_as_bytes(x))
+    wd = helpers.to_device_bytes(helpers.pack_words_as_bytes(w))
+    yd = torch.full((m, n), 0x5A5A5A5A, dtype=torch.int32, device="cuda:0")
+    getattr(lib, f"linear_v{version}_launch")(xd, wd, yd, m, n, k)
+    assert np.array_equal(yd.cpu().numpy(), want)
+
 
 @pytest.mark.parametrize("version", [0, 1, 2, 10, 11, 20, 21])
 def test_reference_entry_points(gpu, version):

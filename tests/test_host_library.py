@@ -86,7 +86,9 @@ def test_kernel_dispatch_table():
     assert lib.kernel_for_shape(64, 4096, 14336) == "skinny"
     assert lib.kernel_for_shape(65, 4096, 4096) == "mfma"
     assert lib.kernel_for_shape(128, 128, 64) == "simple"     # K below one pipeline stage
-    assert lib.kernel_for_shape(128, 128, 200) == "simple"    # K % 128 != 0
+    assert lib.kernel_for_shape(128, 128, 200) == "simple"    # K % 128 != 0, tiny
+    assert lib.kernel_for_shape(1000, 3000, 4104) == "fp6"    # K % 128 != 0: padded by the converter
+    assert lib.kernel_for_shape(16, 4096, 4104) == "fp6"
     assert lib.kernel_for_shape(4, 4, 12) == "invalid"
 
 
@@ -106,7 +108,8 @@ def test_workspace_accounting():
     # caller-owned converted operands: rows padded to 256, 0.75 byte per element
     assert lib.fp6_operand_bytes(8192, 8192) == 8192 * 8192 * 3 // 4
     assert lib.fp6_operand_bytes(1, 128) == 256 * 128 * 3 // 4
-    assert lib.fp6_operand_bytes(16, 200) == 0            # K % 128 != 0
+    assert lib.fp6_operand_bytes(16, 200) == 256 * 256 * 3 // 4   # K padded to 256
+    assert lib.fp6_operand_bytes(16, 12) == 0             # K % 8 != 0
     assert lib.fp6_operand_bytes(16, 1 << 18) == 0        # beyond the exact range
 
 
