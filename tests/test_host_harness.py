@@ -20,7 +20,7 @@ def _binary(name: str) -> Path:
 
 
 def test_harness_binaries_link_against_the_library():
-    for name in ("correctness", "benchmark"):
+    for name in ("correctness", "benchmark", "vendor_compare"):
         out = subprocess.run(["ldd", str(_binary(name))], check=True, capture_output=True, text=True).stdout
         assert "libint4linear.so" in out and "not found" not in out, out
 
@@ -65,3 +65,17 @@ def test_benchmark_harness_reports_tops(gpu):
     assert r.returncode == 0, r.stdout + r.stderr
     lines = re.findall(r"\[PERF\] (\d+)x(\d+)x(\d+) kernel=(\w+) median ([\d.]+) ms .* ([\d.]+) TOPS", r.stdout)
     assert len(lines) == 2 and all(float(l[5]) > 0 for l in lines), r.stdout
+
+
+@pytest.mark.gpu
+def test_vendor_comparison_agrees_bit_for_bit(gpu):
+    """hipBLASLt's int8 GEMM on the widened operands is an independent implementation of the
+    same product: the harness exits non-zero if any output differs."""
+    r = subprocess.run([str(_binary("vendor_compare")), "--iters", "3", "--warmup", "1",
+                        "1024x1024x1024", "300x520x512", "16x4096x4096", "2048x2048x2048"],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout + r.stderr
+    lines = [l for l in r.stdout.splitlines() if l.startswith("[VENDOR]")]
+    assert len(lines) == 4, r.stdout
+    for l in lines:
+        assert "results identical" in l or "offers no int8" in l, l
