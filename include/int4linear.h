@@ -71,6 +71,21 @@ int int4linear_gemm_s4s4s32(const void *a_packed_d, const void *b_packed_d, void
 int int4linear_gemm_s4s4s32_ex(const void *a_packed_d, const void *b_packed_d, void *c_d,
                                int m, int n, int k, int kernel, void *stream);
 
+/* The linear layer with an epilogue fused into the GEMM's store.  The reference has no
+ * such entry point; its README lists the bias add as future work (README.md:72).
+ *   int4linear_linear_s32:  Y[i][j] = sum_l X[i][l] W[j][l] + bias[j]          (int32, wraps)
+ *   int4linear_linear_f32:  Y[i][j] = ((float)(sum + bias[j]) * row_scale[i]) * col_scale[j]
+ * bias_d (n int32), row_scale_d (m floats: per-token activation scale) and col_scale_d
+ * (n floats: per-output-channel weight scale) may each be NULL (0 / 1).  The integer part is
+ * exact; the conversion to float rounds to nearest once and each multiplication once, in
+ * the order written.  `kernel` is an INT4LINEAR_KERNEL_* value; other arguments as for
+ * int4linear_gemm_s4s4s32. */
+int int4linear_linear_s32(const void *x_packed_d, const void *w_packed_d, const int *bias_d, void *y_d,
+                          int m, int n, int k, int kernel, void *stream);
+int int4linear_linear_f32(const void *x_packed_d, const void *w_packed_d, const int *bias_d,
+                          const float *row_scale_d, const float *col_scale_d, float *y_d,
+                          int m, int n, int k, int kernel, void *stream);
+
 /* Device-side counterparts of utils/packer.cpp:3-18 (pack) and :20-31 (unpack):
  * src_d / dst_d are device arrays with the reference's host layouts (m x n ints
  * unpacked, m x ceil(n/8) 32-bit words packed).  Asynchronous on `stream`. */

@@ -11,6 +11,8 @@ from .api import (  # noqa: F401
     gemm_s4s4s32,
     init,
     kernel_for_shape,
+    linear_f32,
+    linear_s32,
     linear_v0_launch,
     linear_v1_launch,
     linear_v2_launch,

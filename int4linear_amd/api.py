@@ -51,6 +51,28 @@ def gemm_s4s4s32(a_packed_d, b_packed_d, c_d, m: int, n: int, k: int, *, kernel:
     _lib.check(st)
 
 
+def linear_s32(x_packed_d, w_packed_d, bias_d, y_d, m: int, n: int, k: int, *, kernel: str = "auto",
+               stream: int | None = None) -> None:
+    """Y = X * W^T + bias (int32); bias_d may be None."""
+    lib = _lib.load()
+    if stream is None:
+        stream = _current_stream()
+    _lib.check(lib.int4linear_linear_s32(_ptr(x_packed_d), _ptr(w_packed_d), _ptr(bias_d), _ptr(y_d), m, n, k,
+                                         KERNELS[kernel], ctypes.c_void_p(stream)))
+
+
+def linear_f32(x_packed_d, w_packed_d, bias_d, row_scale_d, col_scale_d, y_d, m: int, n: int, k: int, *,
+               kernel: str = "auto", stream: int | None = None) -> None:
+    """Y (float32) = ((float)(X * W^T + bias) * row_scale[i]) * col_scale[j]; each of bias_d,
+    row_scale_d, col_scale_d may be None."""
+    lib = _lib.load()
+    if stream is None:
+        stream = _current_stream()
+    _lib.check(lib.int4linear_linear_f32(_ptr(x_packed_d), _ptr(w_packed_d), _ptr(bias_d), _ptr(row_scale_d),
+                                         _ptr(col_scale_d), _ptr(y_d), m, n, k, KERNELS[kernel],
+                                         ctypes.c_void_p(stream)))
+
+
 def fp6_operand_bytes(rows: int, k: int) -> int:
     """Bytes of the converted (FP6) form of a rows x k operand; 0 if k is unsupported."""
     return int(_lib.load().int4linear_fp6_operand_bytes(rows, k))

@@ -118,7 +118,7 @@ int pick_kernel(int m, int n, int k)
 // by the stream; a call on a different stream than the previous user first waits for
 // that user's GEMM to finish with the workspace.
 int run_fp6(PerDevice *pd, const void *a, const void *b, void *c, int m, int n, int k,
-            hipStream_t stream)
+            const Epilogue &ep, hipStream_t stream)
 {
     const size_t need = fp6_workspace_bytes(m, n, k);
     if (need > g_workspace_limit.load())
@@ -151,7 +151,7 @@ int run_fp6(PerDevice *pd, const void *a, const void *b, void *c, int m, int n, 
         if (e != hipSuccess)
             return fail_hip(e);
     }
-    e = launch_fp6(a, b, c, m, n, k, pd->ws, pd->info, stream);
+    e = launch_fp6(a, b, c, m, n, k, pd->ws, ep, pd->info, stream);
     if (e != hipSuccess)
         return fail_hip(e);
     e = hipEventRecord(pd->ws_event, stream);
@@ -163,7 +163,7 @@ int run_fp6(PerDevice *pd, const void *a, const void *b, void *c, int m, int n, 
 }
 
 int gemm_impl(const void *a, const void *b, void *c, int m, int n, int k, int kernel,
-              void *stream_v)
+              void *stream_v, const Epilogue &ep = Epilogue{})
 {
     if (m < 0 || n < 0 || k < 0 || (k % 8) != 0)
         return INT4LINEAR_ERR_SHAPE;
@@ -184,8 +184,13 @@ int gemm_impl(const void *a, const void *b, void *c, int m, int n, int k, int ke
         return st;
     hipStream_t stream = (hipStream_t)stream_v;
 
-    if (k == 0) {
+    const bool plain = !ep.bias && !ep.row_scale && !ep.col_scale && !ep.f32;
+    if (k == 0 && plain) {
         hipError_t e = launch_zero_i32((int *)c, (size_t)m * (size_t)n, stream);
+        return e == hipSuccess ? INT4LINEAR_OK : fail_hip(e);
+    }
+    if (k == 0) {  // empty sum with an epilogue: the scalar kernel's loop runs zero times
+        hipError_t e = launch_simple(a, b, c, m, n, k, ep, stream);
         return e == hipSuccess ? INT4LINEAR_OK : fail_hip(e);
     }
 
@@ -195,7 +200,7 @@ int gemm_impl(const void *a, const void *b, void *c, int m, int n, int k, int ke
     if (kernel == INT4LINEAR_KERNEL_FP6) {
         if (!fp6_supports(m, n, k))
             return INT4LINEAR_ERR_UNSUPPORTED;
-        const int st6 = run_fp6(pd, a, b, c, m, n, k, stream);
+        const int st6 = run_fp6(pd, a, b, c, m, n, k, ep, stream);
         // Under automatic dispatch a workspace that cannot be had falls back to a kernel
         // that needs none.
         if (st6 == INT4LINEAR_OK || !automatic)
@@ -206,24 +211,24 @@ int gemm_impl(const void *a, const void *b, void *c, int m, int n, int k, int ke
     hipError_t e = hipSuccess;
     switch (kernel) {
     case INT4LINEAR_KERNEL_SIMPLE:
-        e = launch_simple(a, b, c, m, n, k, stream);
+        e = launch_simple(a, b, c, m, n, k, ep, stream);
         break;
     case INT4LINEAR_KERNEL_MFMA:
         if (!mfma_supports(m, n, k))
             return INT4LINEAR_ERR_UNSUPPORTED;
-        e = launch_mfma(a, b, c, m, n, k, pd->info, stream);
+        e = launch_mfma(a, b, c, m, n, k, ep, pd->info, stream);
         break;
     case INT4LINEAR_KERNEL_MFMA_128:
     case INT4LINEAR_KERNEL_MFMA_256:
         if (!mfma_supports(m, n, k))
             return INT4LINEAR_ERR_UNSUPPORTED;
-        e = launch_mfma_tile(a, b, c, m, n, k, kernel == INT4LINEAR_KERNEL_MFMA_128 ? 128 : 256, pd->info,
-                             stream);
+        e = launch_mfma_tile(a, b, c, m, n, k, kernel == INT4LINEAR_KERNEL_MFMA_128 ? 128 : 256, ep,
+                             pd->info, stream);
         break;
     case INT4LINEAR_KERNEL_SKINNY:
         if (!skinny_supports(m, n, k))
             return INT4LINEAR_ERR_UNSUPPORTED;
-        e = launch_skinny(a, b, c, m, n, k, pd->info, stream);
+        e = launch_skinny(a, b, c, m, n, k, ep, pd->info, stream);
         break;
     default:
         return INT4LINEAR_ERR_UNSUPPORTED;
@@ -262,6 +267,26 @@ int int4linear_gemm_s4s4s32_ex(const void *a_packed_d, const void *b_packed_d, v
                                int n, int k, int kernel, void *stream)
 {
     return gemm_impl(a_packed_d, b_packed_d, c_d, m, n, k, kernel, stream);
+}
+
+int int4linear_linear_s32(const void *x_packed_d, const void *w_packed_d, const int *bias_d, void *y_d,
+                          int m, int n, int k, int kernel, void *stream)
+{
+    Epilogue ep;
+    ep.bias = bias_d;
+    return gemm_impl(x_packed_d, w_packed_d, y_d, m, n, k, kernel, stream, ep);
+}
+
+int int4linear_linear_f32(const void *x_packed_d, const void *w_packed_d, const int *bias_d,
+                          const float *row_scale_d, const float *col_scale_d, float *y_d, int m, int n,
+                          int k, int kernel, void *stream)
+{
+    Epilogue ep;
+    ep.bias = bias_d;
+    ep.row_scale = row_scale_d;
+    ep.col_scale = col_scale_d;
+    ep.f32 = 1;
+    return gemm_impl(x_packed_d, w_packed_d, y_d, m, n, k, kernel, stream, ep);
 }
 
 int int4linear_pack_s32_to_s4(const int *src_d, int *dst_d, int m, int n, void *stream)
@@ -337,7 +362,7 @@ int int4linear_gemm_fp6_converted(const void *a_conv_d, const void *b_conv_d, vo
     int st = ensure_init(&pd);
     if (st != INT4LINEAR_OK)
         return st;
-    hipError_t e = launch_fp6_gemm(a_conv_d, b_conv_d, c_d, m, n, k, pd->info, (hipStream_t)stream);
+    hipError_t e = launch_fp6_gemm(a_conv_d, b_conv_d, c_d, m, n, k, Epilogue{}, pd->info, (hipStream_t)stream);
     return e == hipSuccess ? INT4LINEAR_OK : fail_hip(e);
 }
 

@@ -6,6 +6,31 @@
 
 namespace int4linear {
 
+// Optional work between the accumulator and the store of every output element (i, j):
+//   v = acc + bias[j]                                   (bias null: + 0)
+//   f32 == 0: C is int32 and receives v
+//   f32 != 0: C is float and receives (float)v * row_scale[i] * col_scale[j]
+//             (a null scale counts as 1; the two multiplications happen in that order)
+// Passed to the kernels by value; an all-zero struct is the plain GEMM.
+struct Epilogue {
+    const int32_t *bias = nullptr;
+    const float *row_scale = nullptr;
+    const float *col_scale = nullptr;
+    int f32 = 0;
+};
+
+#if defined(__HIPCC__)
+// The 32 bits stored for one output element.
+__device__ __forceinline__ int epilogue_value(const Epilogue &ep, int acc, int bias_j, float row_scale_i,
+                                              float col_scale_j)
+{
+    const int v = acc + bias_j;
+    if (!ep.f32)
+        return v;
+    return __float_as_int(((float)v * row_scale_i) * col_scale_j);
+}
+#endif
+
 struct DeviceInfo {
     int cu_count = 0;      // compute units on the device
     int lds_per_cu = 0;    // bytes of LDS a workgroup may use
@@ -13,17 +38,17 @@ struct DeviceInfo {
 
 // One thread per output, scalar nibble decode.  Any M, N >= 1 and K % 8 == 0.
 hipError_t launch_simple(const void *a, const void *b, void *c, int m, int n, int k,
-                         hipStream_t stream);
+                         const Epilogue &ep, hipStream_t stream);
 
 // LDS-pipelined MFMA kernel.  Requires K % 128 == 0, K >= 128.
 bool mfma_supports(int m, int n, int k);
 hipError_t mfma_init(const DeviceInfo &dev);
 hipError_t launch_mfma(const void *a, const void *b, void *c, int m, int n, int k,
-                       const DeviceInfo &dev, hipStream_t stream);
+                       const Epilogue &ep, const DeviceInfo &dev, hipStream_t stream);
 
 // The same kernel with the workgroup tile forced to 128 x 128 or 256 x 256 (`tile`).
 hipError_t launch_mfma_tile(const void *a, const void *b, void *c, int m, int n, int k, int tile,
-                            const DeviceInfo &dev, hipStream_t stream);
+                            const Epilogue &ep, const DeviceInfo &dev, hipStream_t stream);
 
 // FP6-MFMA path: converts both operands into a workspace of fp6_workspace_bytes() bytes
 // (256-byte aligned), then runs the GEMM on it.  Requires K % 128 == 0, K < 2^18.
@@ -35,15 +60,15 @@ hipError_t fp6_init(const DeviceInfo &dev);
 size_t fp6_operand_bytes(int rows, int k);
 hipError_t launch_fp6_convert(const void *src, void *dst, int rows, int k, hipStream_t stream);
 hipError_t launch_fp6_gemm(const void *a_conv, const void *b_conv, void *c, int m, int n, int k,
-                           const DeviceInfo &dev, hipStream_t stream);
+                           const Epilogue &ep, const DeviceInfo &dev, hipStream_t stream);
 hipError_t launch_fp6(const void *a, const void *b, void *c, int m, int n, int k, void *workspace,
-                      const DeviceInfo &dev, hipStream_t stream);
+                      const Epilogue &ep, const DeviceInfo &dev, hipStream_t stream);
 
 // Weight-streaming kernel for skinny M.  Requires M <= 64, K % 128 == 0.
 bool skinny_supports(int m, int n, int k);
 hipError_t skinny_init(const DeviceInfo &dev);
 hipError_t launch_skinny(const void *a, const void *b, void *c, int m, int n, int k,
-                         const DeviceInfo &dev, hipStream_t stream);
+                         const Epilogue &ep, const DeviceInfo &dev, hipStream_t stream);
 
 // Device packer / unpacker, utils/packer.cpp layouts.
 hipError_t launch_pack(const int *src, int *dst, int m, int n, hipStream_t stream);

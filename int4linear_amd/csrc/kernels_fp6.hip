@@ -231,7 +231,7 @@ struct Fp6Config {
 template <class C>
 __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
     const uint8_t *__restrict__ XW, const uint8_t *__restrict__ WW, int32_t *__restrict__ Y,
-    int M, int N, int K, int tiles_m, int tiles_n)
+    int M, int N, int K, int tiles_m, int tiles_n, Epilogue ep)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
@@ -243,6 +243,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
     const int total_tiles = tiles_m * tiles_n;
     const int nblk = gridDim.x;
     const int bid = blockIdx.x;
+    const bool ep_plain = !ep.bias && !ep.row_scale && !ep.col_scale && !ep.f32;
     if (bid >= total_tiles)
         return;
     const int my_tiles = (total_tiles - bid + nblk - 1) / nblk;
@@ -444,16 +445,51 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
                 const int ncol = ln + i * kFragRows;
                 col_off[i] = ncol < cols_left ? (unsigned)ncol * 4u : 0x40000000u;
             }
+            if (ep_plain) {
 #pragma unroll
-            for (int j = 0; j < C::FM; ++j) {
+                for (int j = 0; j < C::FM; ++j) {
 #pragma unroll
-                for (int t = 0; t < 16; ++t) {
-                    const int dm = j * kFragRows + 8 * (t / 4) + (t % 4);  // uniform
-                    const unsigned row_off = lm + dm < rows_left ? lm_off + (unsigned)dm * (unsigned)N * 4u : 0x80000000u;
+                    for (int t = 0; t < 16; ++t) {
+                        const int dm = j * kFragRows + 8 * (t / 4) + (t % 4);  // uniform
+                        const unsigned row_off = lm + dm < rows_left ? lm_off + (unsigned)dm * (unsigned)N * 4u : 0x80000000u;
 #pragma unroll
-                    for (int i = 0; i < C::FN; ++i) {
-                        const int v = (int)acc[i][j][t];  // exact: the accumulator holds an integer
-                        __builtin_amdgcn_raw_buffer_store_b32((unsigned)v, rsrc, row_off + col_off[i], 0, 2 /* nt */);
+                        for (int i = 0; i < C::FN; ++i) {
+                            const int v = (int)acc[i][j][t];
+                            __builtin_amdgcn_raw_buffer_store_b32((unsigned)v, rsrc, row_off + col_off[i], 0, 2 /* nt */);
+                        }
+                    }
+                }
+            } else {
+                // Epilogue operands of this lane's columns and rows (clamped inside the
+                // matrix).  These ordinary loads make the compiler wait for everything in
+                // flight, prefetched stages included: the price of an epilogue, kept out of
+                // the plain path above.
+                int bias_v[C::FN];
+                float cs_v[C::FN];
+#pragma unroll
+                for (int i = 0; i < C::FN; ++i) {
+                    const int ncol = ln + i * kFragRows;
+                    const int nn = n0 + (ncol < cols_left ? ncol : cols_left - 1);
+                    bias_v[i] = ep.bias ? ep.bias[nn] : 0;
+                    cs_v[i] = ep.col_scale ? ep.col_scale[nn] : 1.f;
+                }
+#pragma unroll
+                for (int j = 0; j < C::FM; ++j) {
+                    float rs[16];
+#pragma unroll
+                    for (int t = 0; t < 16; ++t) {
+                        const int dm = j * kFragRows + 8 * (t / 4) + (t % 4);
+                        rs[t] = ep.row_scale ? ep.row_scale[m0 + (lm + dm < rows_left ? lm + dm : rows_left - 1)] : 1.f;
+                    }
+#pragma unroll
+                    for (int t = 0; t < 16; ++t) {
+                        const int dm = j * kFragRows + 8 * (t / 4) + (t % 4);  // uniform
+                        const unsigned row_off = lm + dm < rows_left ? lm_off + (unsigned)dm * (unsigned)N * 4u : 0x80000000u;
+#pragma unroll
+                        for (int i = 0; i < C::FN; ++i) {
+                            const int v = epilogue_value(ep, (int)acc[i][j][t], bias_v[i], rs[t], cs_v[i]);
+                            __builtin_amdgcn_raw_buffer_store_b32((unsigned)v, rsrc, row_off + col_off[i], 0, 2 /* nt */);
+                        }
                     }
                 }
             }
@@ -530,7 +566,7 @@ hipError_t launch_fp6_convert(const void *src, void *dst, int rows, int k, hipSt
 }
 
 hipError_t launch_fp6_gemm(const void *a_conv, const void *b_conv, void *c, int m, int n, int k,
-                           const DeviceInfo &dev, hipStream_t stream)
+                           const Epilogue &ep, const DeviceInfo &dev, hipStream_t stream)
 {
     using C = Fp6Cfg;
     const int tiles_m = (m + kTileRows - 1) / kTileRows;
@@ -542,18 +578,18 @@ hipError_t launch_fp6_gemm(const void *a_conv, const void *b_conv, void *c, int 
     if (grid > total)
         grid = total;
     fp6_gemm_kernel<C><<<(unsigned)grid, C::THREADS, kLdsBytes, stream>>>(
-        (const uint8_t *)a_conv, (const uint8_t *)b_conv, (int32_t *)c, m, n, padded_k(k), tiles_m, tiles_n);
+        (const uint8_t *)a_conv, (const uint8_t *)b_conv, (int32_t *)c, m, n, padded_k(k), tiles_m, tiles_n, ep);
     return hipGetLastError();
 }
 
 hipError_t launch_fp6(const void *a, const void *b, void *c, int m, int n, int k, void *workspace,
-                      const DeviceInfo &dev, hipStream_t stream)
+                      const Epilogue &ep, const DeviceInfo &dev, hipStream_t stream)
 {
     uint8_t *xws = (uint8_t *)workspace;
     uint8_t *wws = xws + operand_ws_bytes(m, k);
     hipError_t e = launch_convert_jobs(make_job(a, xws, m), make_job(b, wws, n), k, stream);
     if (e == hipSuccess)
-        e = launch_fp6_gemm(xws, wws, c, m, n, k, dev, stream);
+        e = launch_fp6_gemm(xws, wws, c, m, n, k, ep, dev, stream);
     return e;
 }
 

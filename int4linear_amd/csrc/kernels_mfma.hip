@@ -130,7 +130,7 @@ __device__ __forceinline__ void tile_coords(int v, int total, int tiles_m, int t
 template <class C>
 __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
     const uint8_t *__restrict__ X, const uint8_t *__restrict__ W, int32_t *__restrict__ Y,
-    int M, int N, int K, int tiles_m, int tiles_n)
+    int M, int N, int K, int tiles_m, int tiles_n, Epilogue ep)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
@@ -143,6 +143,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
     const int total_tiles = tiles_m * tiles_n;
     const int nblk = gridDim.x;
     const int bid = blockIdx.x;
+    const bool ep_plain = !ep.bias && !ep.row_scale && !ep.col_scale && !ep.f32;
     if (bid >= total_tiles)
         return;
     const int my_tiles = (total_tiles - bid + nblk - 1) / nblk;
@@ -476,16 +477,51 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
                 const int ncol = ln + i * kFrag;
                 col_off[i] = ncol < cols_left ? (unsigned)ncol * 4u : 0x40000000u;
             }
+            if (ep_plain) {
 #pragma unroll
-            for (int j = 0; j < C::FM; ++j) {
+                for (int j = 0; j < C::FM; ++j) {
 #pragma unroll
-                for (int t = 0; t < 16; ++t) {
-                    const int dm = j * kFrag + 8 * (t / 4) + (t % 4);   // uniform
-                    const unsigned row_off = lm + dm < rows_left ? lm_off + (unsigned)dm * (unsigned)N * 4u : 0x80000000u;
+                    for (int t = 0; t < 16; ++t) {
+                        const int dm = j * kFrag + 8 * (t / 4) + (t % 4);  // uniform
+                        const unsigned row_off = lm + dm < rows_left ? lm_off + (unsigned)dm * (unsigned)N * 4u : 0x80000000u;
 #pragma unroll
-                    for (int i = 0; i < C::FN; ++i) {
-                        const int v = acc[i][j][t] >> 8;
-                        __builtin_amdgcn_raw_buffer_store_b32((unsigned)v, rsrc, row_off + col_off[i], 0, I4L_STORE_AUX);
+                        for (int i = 0; i < C::FN; ++i) {
+                            const int v = acc[i][j][t] >> 8;
+                            __builtin_amdgcn_raw_buffer_store_b32((unsigned)v, rsrc, row_off + col_off[i], 0, I4L_STORE_AUX);
+                        }
+                    }
+                }
+            } else {
+                // Epilogue operands of this lane's columns and rows (clamped inside the
+                // matrix).  These ordinary loads make the compiler wait for everything in
+                // flight, prefetched stages included: the price of an epilogue, kept out of
+                // the plain path above.
+                int bias_v[C::FN];
+                float cs_v[C::FN];
+#pragma unroll
+                for (int i = 0; i < C::FN; ++i) {
+                    const int ncol = ln + i * kFrag;
+                    const int nn = n0 + (ncol < cols_left ? ncol : cols_left - 1);
+                    bias_v[i] = ep.bias ? ep.bias[nn] : 0;
+                    cs_v[i] = ep.col_scale ? ep.col_scale[nn] : 1.f;
+                }
+#pragma unroll
+                for (int j = 0; j < C::FM; ++j) {
+                    float rs[16];
+#pragma unroll
+                    for (int t = 0; t < 16; ++t) {
+                        const int dm = j * kFrag + 8 * (t / 4) + (t % 4);
+                        rs[t] = ep.row_scale ? ep.row_scale[m0 + (lm + dm < rows_left ? lm + dm : rows_left - 1)] : 1.f;
+                    }
+#pragma unroll
+                    for (int t = 0; t < 16; ++t) {
+                        const int dm = j * kFrag + 8 * (t / 4) + (t % 4);  // uniform
+                        const unsigned row_off = lm + dm < rows_left ? lm_off + (unsigned)dm * (unsigned)N * 4u : 0x80000000u;
+#pragma unroll
+                        for (int i = 0; i < C::FN; ++i) {
+                            const int v = epilogue_value(ep, acc[i][j][t] >> 8, bias_v[i], rs[t], cs_v[i]);
+                            __builtin_amdgcn_raw_buffer_store_b32((unsigned)v, rsrc, row_off + col_off[i], 0, I4L_STORE_AUX);
+                        }
                     }
                 }
             }
@@ -511,7 +547,7 @@ hipError_t set_lds_limit()
 
 template <class C>
 hipError_t launch_cfg(const void *a, const void *b, void *c, int m, int n, int k,
-                      const DeviceInfo &dev, hipStream_t stream)
+                      const Epilogue &ep, const DeviceInfo &dev, hipStream_t stream)
 {
     const int tiles_m = (m + C::BM - 1) / C::BM;
     const int tiles_n = (n + C::BN - 1) / C::BN;
@@ -525,7 +561,7 @@ hipError_t launch_cfg(const void *a, const void *b, void *c, int m, int n, int k
     if ((size_t)C::BM * (size_t)n * 4u > 0x40000000ull)
         return hipErrorInvalidValue;
     mfma_gemm_kernel<C><<<(unsigned)grid, C::THREADS, C::LDS_BYTES, stream>>>(
-        (const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k, tiles_m, tiles_n);
+        (const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k, tiles_m, tiles_n, ep);
     return hipGetLastError();
 }
 
@@ -549,24 +585,24 @@ hipError_t mfma_init(const DeviceInfo &dev)
 }
 
 hipError_t launch_mfma_tile(const void *a, const void *b, void *c, int m, int n, int k, int tile,
-                            const DeviceInfo &dev, hipStream_t stream)
+                            const Epilogue &ep, const DeviceInfo &dev, hipStream_t stream)
 {
     if (tile == 256)
-        return launch_cfg<CfgLarge>(a, b, c, m, n, k, dev, stream);
+        return launch_cfg<CfgLarge>(a, b, c, m, n, k, ep, dev, stream);
     if (tile == 128)
-        return launch_cfg<CfgMedium>(a, b, c, m, n, k, dev, stream);
+        return launch_cfg<CfgMedium>(a, b, c, m, n, k, ep, dev, stream);
     return hipErrorInvalidValue;
 }
 
 hipError_t launch_mfma(const void *a, const void *b, void *c, int m, int n, int k,
-                       const DeviceInfo &dev, hipStream_t stream)
+                       const Epilogue &ep, const DeviceInfo &dev, hipStream_t stream)
 {
     const long tiles_large = (long)((m + CfgLarge::BM - 1) / CfgLarge::BM) *
                              ((n + CfgLarge::BN - 1) / CfgLarge::BN);
     // Use the big tile once it alone can occupy every CU.
     if (tiles_large >= dev.cu_count)
-        return launch_cfg<CfgLarge>(a, b, c, m, n, k, dev, stream);
-    return launch_cfg<CfgMedium>(a, b, c, m, n, k, dev, stream);
+        return launch_cfg<CfgLarge>(a, b, c, m, n, k, ep, dev, stream);
+    return launch_cfg<CfgMedium>(a, b, c, m, n, k, ep, dev, stream);
 }
 
 }  // namespace int4linear

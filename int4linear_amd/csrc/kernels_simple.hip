@@ -21,7 +21,7 @@ __device__ __forceinline__ int nibble_s4(uint32_t word, int slot)
 // LDS one 128-nibble chunk at a time.  test/test_correctness.cu:12-19 semantics.
 __global__ __launch_bounds__(kTile *kTile) void simple_gemm_kernel(
     const uint32_t *__restrict__ a, const uint32_t *__restrict__ b, int32_t *__restrict__ c,
-    int m, int n, int k_words)
+    int m, int n, int k_words, Epilogue ep)
 {
     __shared__ uint32_t a_lds[kTile][kChunkWords + 1];
     __shared__ uint32_t b_lds[kTile][kChunkWords + 1];
@@ -49,7 +49,9 @@ __global__ __launch_bounds__(kTile *kTile) void simple_gemm_kernel(
         __syncthreads();
     }
     if (row < m && col < n)
-        c[row * n + col] = acc;
+        c[row * n + col] = epilogue_value(ep, acc, ep.bias ? ep.bias[col] : 0,
+                                          ep.row_scale ? ep.row_scale[row] : 1.f,
+                                          ep.col_scale ? ep.col_scale[col] : 1.f);
 }
 
 // utils/packer.cpp:3-18 on device arrays: one thread per destination word.
@@ -96,13 +98,13 @@ __global__ void zero_i32_kernel(int4 *__restrict__ dst4, int *__restrict__ dst, 
 }  // namespace
 
 hipError_t launch_simple(const void *a, const void *b, void *c, int m, int n, int k,
-                         hipStream_t stream)
+                         const Epilogue &ep, hipStream_t stream)
 {
     dim3 grid((n + kTile - 1) / kTile, (m + kTile - 1) / kTile);
     if (grid.y > 65535u)
         return hipErrorInvalidValue;
     simple_gemm_kernel<<<grid, kTile * kTile, 0, stream>>>(
-        (const uint32_t *)a, (const uint32_t *)b, (int32_t *)c, m, n, k / 8);
+        (const uint32_t *)a, (const uint32_t *)b, (int32_t *)c, m, n, k / 8, ep);
     return hipGetLastError();
 }
 

@@ -92,7 +92,7 @@ template <int T, int R, int FMX, bool XDMA>
 __global__ __launch_bounds__(1024) void skinny_kernel(const uint8_t *__restrict__ X,
                                                       const uint8_t *__restrict__ W,
                                                       int32_t *__restrict__ Y, int M, int N, int K,
-                                                      int rows_blk)
+                                                      int rows_blk, Epilogue ep)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int kWaveTiles = T * (R + (XDMA ? FMX : 0));
@@ -237,6 +237,13 @@ __global__ __launch_bounds__(1024) void skinny_kernel(const uint8_t *__restrict_
         const int m = f * 16 + fr;
         const int n = n0 + rg * 16 + 4 * fg;
         if (m < M) {
+            const float rs = ep.row_scale ? ep.row_scale[m] : 1.f;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int nn = n + q < n_end ? n + q : n_end - 1;
+                sum[q] = epilogue_value(ep, sum[q], ep.bias ? ep.bias[nn] : 0, rs,
+                                        ep.col_scale ? ep.col_scale[nn] : 1.f);
+            }
             int32_t *dst = Y + (size_t)m * N + n;
             if (n + 3 < n_end && (N & 3) == 0) {
                 *(v4i *)dst = sum;
@@ -255,7 +262,7 @@ __global__ __launch_bounds__(1024) void skinny_kernel(const uint8_t *__restrict_
 template <int FMX, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void skinny_basic_kernel(
     const uint8_t *__restrict__ X, const uint8_t *__restrict__ W, int32_t *__restrict__ Y,
-    int M, int N, int K)
+    int M, int N, int K, Epilogue ep)
 {
     __shared__ v4i partial[WAVES][FMX][64];
     const int lane = threadIdx.x & 63;
@@ -304,6 +311,13 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_basic_kernel(
         const int m = f * 16 + (l & 15);
         const int n = n0 + 4 * (l >> 4);
         if (m < M) {
+            const float rs = ep.row_scale ? ep.row_scale[m] : 1.f;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int nn = n + q < N ? n + q : N - 1;
+                s[q] = epilogue_value(ep, s[q], ep.bias ? ep.bias[nn] : 0, rs,
+                                      ep.col_scale ? ep.col_scale[nn] : 1.f);
+            }
             int32_t *dst = Y + (size_t)m * N + n;
             if (n + 3 < N && (N & 3) == 0) {
                 *(v4i *)dst = s;
@@ -319,16 +333,16 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_basic_kernel(
 
 template <int FMX>
 hipError_t launch_basic(const void *a, const void *b, void *c, int m, int n, int k,
-                        hipStream_t stream)
+                        const Epilogue &ep, hipStream_t stream)
 {
     const unsigned grid = (unsigned)((n + 15) / 16);
     const int steps = k / 128;
     if (steps >= 8)
         skinny_basic_kernel<FMX, 8><<<grid, 512, 0, stream>>>((const uint8_t *)a, (const uint8_t *)b,
-                                                              (int32_t *)c, m, n, k);
+                                                              (int32_t *)c, m, n, k, ep);
     else
         skinny_basic_kernel<FMX, 2><<<grid, 128, 0, stream>>>((const uint8_t *)a, (const uint8_t *)b,
-                                                              (int32_t *)c, m, n, k);
+                                                              (int32_t *)c, m, n, k, ep);
     return hipGetLastError();
 }
 
@@ -394,9 +408,9 @@ bool make_plan(int m, int n, int k, int cu_count, Plan &p)
 
 template <int T, int R, int FMX, bool XDMA>
 hipError_t launch_plan(const Plan &p, const void *a, const void *b, void *c, int m, int n, int k,
-                       hipStream_t stream)
+                       const Epilogue &ep, hipStream_t stream)
 {
-    if constexpr (!XDMA && FMX > 2) {
+    if constexpr (!XDMA && (FMX > 2 || R > 1)) {  // the register-X variant is only ever planned with R == 1
         return p.s == 0 ? hipSuccess : hipErrorInvalidConfiguration;  // never planned
     } else {
     auto kern = skinny_kernel<T, R, FMX, XDMA>;
@@ -404,18 +418,18 @@ hipError_t launch_plan(const Plan &p, const void *a, const void *b, void *c, int
         return hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
     const unsigned grid = (unsigned)((n + p.rows_blk - 1) / p.rows_blk);
     kern<<<grid, p.s * 64, p.lds, stream>>>((const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k,
-                                            p.rows_blk);
+                                            p.rows_blk, ep);
     return hipGetLastError();
     }
 }
 
 template <int T, bool XDMA>
 hipError_t dispatch_rf(const Plan &p, const void *a, const void *b, void *c, int m, int n, int k,
-                       hipStream_t stream)
+                       const Epilogue &ep, hipStream_t stream)
 {
 #define I4L_CASE(R_, F_)                                                      \
     if (p.r == R_ && p.fmx == F_)                                             \
-        return launch_plan<T, R_, F_, XDMA>(p, a, b, c, m, n, k, stream);
+        return launch_plan<T, R_, F_, XDMA>(p, a, b, c, m, n, k, ep, stream);
     I4L_CASE(4, 1)
     I4L_CASE(2, 1)
     I4L_CASE(1, 1)
@@ -438,15 +452,15 @@ hipError_t skinny_init(const DeviceInfo &)
         p.s = 0;
         p.r = rf[0];
         p.fmx = rf[1];
-        hipError_t e = dispatch_rf<1, true>(p, nullptr, nullptr, nullptr, 0, 0, 0, nullptr);
+        hipError_t e = dispatch_rf<1, true>(p, nullptr, nullptr, nullptr, 0, 0, 0, Epilogue{}, nullptr);
         if (e == hipSuccess)
-            e = dispatch_rf<2, true>(p, nullptr, nullptr, nullptr, 0, 0, 0, nullptr);
+            e = dispatch_rf<2, true>(p, nullptr, nullptr, nullptr, 0, 0, 0, Epilogue{}, nullptr);
         if (e == hipSuccess)
-            e = dispatch_rf<3, true>(p, nullptr, nullptr, nullptr, 0, 0, 0, nullptr);
+            e = dispatch_rf<3, true>(p, nullptr, nullptr, nullptr, 0, 0, 0, Epilogue{}, nullptr);
         if (e == hipSuccess)
-            e = dispatch_rf<4, true>(p, nullptr, nullptr, nullptr, 0, 0, 0, nullptr);
+            e = dispatch_rf<4, true>(p, nullptr, nullptr, nullptr, 0, 0, 0, Epilogue{}, nullptr);
         if (e == hipSuccess)
-            e = dispatch_rf<4, false>(p, nullptr, nullptr, nullptr, 0, 0, 0, nullptr);
+            e = dispatch_rf<4, false>(p, nullptr, nullptr, nullptr, 0, 0, 0, Epilogue{}, nullptr);
         if (e != hipSuccess)
             return e;
     }
@@ -459,32 +473,32 @@ bool skinny_supports(int m, int n, int k)
 }
 
 hipError_t launch_skinny(const void *a, const void *b, void *c, int m, int n, int k,
-                         const DeviceInfo &dev, hipStream_t stream)
+                         const Epilogue &ep, const DeviceInfo &dev, hipStream_t stream)
 {
     Plan p;
     if (make_plan(m, n, k, dev.cu_count, p)) {
         if (!p.xdma)
-            return dispatch_rf<4, false>(p, a, b, c, m, n, k, stream);
+            return dispatch_rf<4, false>(p, a, b, c, m, n, k, ep, stream);
         switch (p.t) {
         case 1:
-            return dispatch_rf<1, true>(p, a, b, c, m, n, k, stream);
+            return dispatch_rf<1, true>(p, a, b, c, m, n, k, ep, stream);
         case 2:
-            return dispatch_rf<2, true>(p, a, b, c, m, n, k, stream);
+            return dispatch_rf<2, true>(p, a, b, c, m, n, k, ep, stream);
         case 3:
-            return dispatch_rf<3, true>(p, a, b, c, m, n, k, stream);
+            return dispatch_rf<3, true>(p, a, b, c, m, n, k, ep, stream);
         default:
-            return dispatch_rf<4, true>(p, a, b, c, m, n, k, stream);
+            return dispatch_rf<4, true>(p, a, b, c, m, n, k, ep, stream);
         }
     }
     switch ((m + 15) / 16) {
     case 1:
-        return launch_basic<1>(a, b, c, m, n, k, stream);
+        return launch_basic<1>(a, b, c, m, n, k, ep, stream);
     case 2:
-        return launch_basic<2>(a, b, c, m, n, k, stream);
+        return launch_basic<2>(a, b, c, m, n, k, ep, stream);
     case 3:
-        return launch_basic<3>(a, b, c, m, n, k, stream);
+        return launch_basic<3>(a, b, c, m, n, k, ep, stream);
     default:
-        return launch_basic<4>(a, b, c, m, n, k, stream);
+        return launch_basic<4>(a, b, c, m, n, k, ep, stream);
     }
 }
 

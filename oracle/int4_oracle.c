@@ -18,6 +18,12 @@
  *                        algebraic invariants (linearity, K-permutation,
  *                        transposition) and pure-Python brute force on tiny shapes.
  *   oracle_is_same     - trivial; checked on equal / one-element-different arrays.
+ *   oracle_epilogue    - not in the reference's code (its README.md:72 names the bias
+ *                        add as future work); the definition is this library's own
+ *                        header.  Pinned against numpy: int32 wrap-around add for the
+ *                        bias, float32 astype / multiply (IEEE round-to-nearest, same
+ *                        order) for the scaled output, plus the identities
+ *                        "no operands == the plain product" and "scales of 1 == cast".
  */
 #include <stddef.h>
 #include <stdint.h>
@@ -101,4 +107,28 @@ int oracle_is_same(const int *a, const int *b, int count)
         if (a[i] != b[i])
             return 0;
     return 1;
+}
+
+/* The epilogue of int4linear_linear_s32 / _f32, applied in place to a finished int32
+ * product y (m x n): v = y[i][j] + bias[j] (two's-complement wrap), and for f32 != 0
+ * the 32 bits of ((float)v * row_scale[i]) * col_scale[j].  Null operands count as 0 / 1.
+ * Compiled without floating-point contraction; the two products round separately. */
+void oracle_epilogue(int *y, int m, int n, const int *bias, const float *row_scale,
+                     const float *col_scale, int f32)
+{
+    for (int i = 0; i < m; ++i) {
+        const float rs = row_scale ? row_scale[i] : 1.0f;
+        for (int j = 0; j < n; ++j) {
+            const uint32_t sum = (uint32_t)y[(size_t)i * n + j] + (uint32_t)(bias ? bias[j] : 0);
+            int v = (int)sum;
+            if (f32) {
+                volatile float a = (float)v * rs;  /* volatile: no fused or reassociated product */
+                const float f = a * (col_scale ? col_scale[j] : 1.0f);
+                union { float f; int i; } u;
+                u.f = f;
+                v = u.i;
+            }
+            y[(size_t)i * n + j] = v;
+        }
+    }
 }

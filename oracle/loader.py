@@ -91,6 +91,30 @@ def linear_ref(x: np.ndarray, w: np.ndarray, threads: int = 1) -> np.ndarray:
     return y
 
 
+def epilogue(y: np.ndarray, bias=None, row_scale=None, col_scale=None, f32: bool = False) -> np.ndarray:
+    """Applies the linear layer's epilogue to an int32 product; returns int32, or float32
+    when f32 is set."""
+    out = np.ascontiguousarray(_i32(y)).copy()
+    m, n = out.shape
+    keep = []
+
+    def ptr(a, dtype, count):
+        if a is None:
+            return None
+        a = np.ascontiguousarray(a, dtype=dtype)
+        assert a.size == count
+        keep.append(a)
+        return a.ctypes.data
+
+    fn = oracle().oracle_epilogue
+    fn.restype = None
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                   ctypes.c_int]
+    fn(out.ctypes.data, m, n, ptr(bias, np.int32, n), ptr(row_scale, np.float32, m), ptr(col_scale, np.float32, n),
+       1 if f32 else 0)
+    return out.view(np.float32) if f32 else out
+
+
 def is_same(a: np.ndarray, b: np.ndarray) -> bool:
     a = _i32(a).ravel()
     b = _i32(b).ravel()

@@ -2,7 +2,11 @@
 // launches, 50 timed ones, every timed launch preceded by a cache-cleaning fill and bracketed
 // by its own event pair, median reported as 2*M*N*K / t in TOPS ("[PERF] ... TOPS").
 //
-//   benchmark [--kernel auto|simple|mfma|mfma128|mfma256|skinny|fp6] [--iters I] [--warmup W] [--no-flush] MxNxK ...
+//   benchmark [--kernel auto|simple|mfma|mfma128|mfma256|skinny|fp6] [--epilogue none|bias|f32]
+//             [--iters I] [--warmup W] [--no-flush] MxNxK ...
+//
+// --epilogue bias times int4linear_linear_s32 (bias add fused into the store), f32 times
+// int4linear_linear_f32 (bias, per-row and per-column scales, float output).
 //
 // The reference cleans twice its L2 (benchmark.cu:77-91); an MI355X also has a 256 MiB
 // memory-side cache behind the eight L2s, so the fill here is 512 MiB.  Operand values are
@@ -30,7 +34,7 @@ int kernel_id(const std::string &name)
 
 int main(int argc, char **argv)
 {
-    std::string kernel = "auto";
+    std::string kernel = "auto", epilogue = "none";
     int iters = 50, warmup = 5;
     bool flush = true;
     std::vector<Shape> shapes;
@@ -38,6 +42,7 @@ int main(int argc, char **argv)
         const std::string a = argv[i];
         Shape s;
         if (a == "--kernel" && i + 1 < argc) kernel = argv[++i];
+        else if (a == "--epilogue" && i + 1 < argc) epilogue = argv[++i];
         else if (a == "--iters" && i + 1 < argc) iters = std::atoi(argv[++i]);
         else if (a == "--warmup" && i + 1 < argc) warmup = std::atoi(argv[++i]);
         else if (a == "--no-flush") flush = false;
@@ -49,8 +54,8 @@ int main(int argc, char **argv)
         }
     }
     const int kid = kernel_id(kernel);
-    if (kid < 0 || iters < 1) {
-        std::fprintf(stderr, "bad --kernel or --iters\n");
+    if (kid < 0 || iters < 1 || (epilogue != "none" && epilogue != "bias" && epilogue != "f32")) {
+        std::fprintf(stderr, "bad --kernel, --epilogue or --iters\n");
         return 2;
     }
     if (shapes.empty()) shapes.push_back({8192, 8192, 8192});
@@ -68,8 +73,27 @@ int main(int argc, char **argv)
         upload_packed(uniform_s4(11, (size_t)m * k), m, k, xd);
         upload_packed(uniform_s4(12, (size_t)n * k), n, k, wd);
 
+        DeviceBuffer bias((size_t)n * sizeof(int)), rscale((size_t)m * sizeof(float)), cscale((size_t)n * sizeof(float));
+        {
+            std::vector<int> b((size_t)n);
+            std::vector<float> r((size_t)m), c((size_t)n);
+            Rng rng(13);
+            for (auto &v : b) v = (int)(rng.next() % 2001) - 1000;
+            for (auto &v : r) v = (float)(0.01 + rng.unit());
+            for (auto &v : c) v = (float)(0.01 + rng.unit());
+            HIP_OK(hipMemcpy(bias.p, b.data(), bias.bytes, hipMemcpyHostToDevice));
+            HIP_OK(hipMemcpy(rscale.p, r.data(), rscale.bytes, hipMemcpyHostToDevice));
+            HIP_OK(hipMemcpy(cscale.p, c.data(), cscale.bytes, hipMemcpyHostToDevice));
+        }
         auto launch = [&]() {
-            const int st = int4linear_gemm_s4s4s32_ex(xd.p, wd.p, yd.p, m, n, k, kid, nullptr);
+            int st;
+            if (epilogue == "bias")
+                st = int4linear_linear_s32(xd.p, wd.p, (const int *)bias.p, yd.p, m, n, k, kid, nullptr);
+            else if (epilogue == "f32")
+                st = int4linear_linear_f32(xd.p, wd.p, (const int *)bias.p, (const float *)rscale.p,
+                                           (const float *)cscale.p, (float *)yd.p, m, n, k, kid, nullptr);
+            else
+                st = int4linear_gemm_s4s4s32_ex(xd.p, wd.p, yd.p, m, n, k, kid, nullptr);
             if (st != INT4LINEAR_OK) {
                 std::fprintf(stderr, "[%dx%dx%d] %s\n", m, n, k, int4linear_status_string(st));
                 std::exit(2);
@@ -94,9 +118,9 @@ int main(int argc, char **argv)
         const double median_ms = ms[(size_t)iters / 2];
         const double ops = 2.0 * m * (double)n * k;
         const double bytes = (double)m * k / 2 + (double)n * k / 2 + 4.0 * m * n;
-        std::printf("[PERF] %dx%dx%d kernel=%s median %.4f ms (min %.4f)  %lf TOPS  %.1f GB/s\n", m, n, k,
+        std::printf("[PERF] %dx%dx%d kernel=%s epilogue=%s median %.4f ms (min %.4f)  %lf TOPS  %.1f GB/s\n", m, n, k,
                     kid == INT4LINEAR_KERNEL_AUTO ? int4linear_kernel_for_shape(m, n, k) : kernel.c_str(),
-                    median_ms, (double)ms[0], ops / (median_ms * 1e9), bytes / (median_ms * 1e6));
+                    epilogue.c_str(), median_ms, (double)ms[0], ops / (median_ms * 1e9), bytes / (median_ms * 1e6));
     }
     HIP_OK(hipEventDestroy(start));
     HIP_OK(hipEventDestroy(stop));

@@ -156,6 +156,48 @@ def test_ragged_k_runs_on_the_fp6_kernel(gpu, host_threads, m, n, k):
         assert np.array_equal(got, want), kern
 
 
+# ---- epilogue: bias add and scaled float output, fused into every kernel's store ----------
+
+@pytest.mark.parametrize("m, n, k, kernels", [
+    (300, 520, 512, ("auto", "simple", "mfma128", "mfma256", "fp6")),
+    (16, 1024, 1024, ("auto", "skinny", "mfma", "fp6")),
+    (40, 515, 14336, ("skinny",)),
+    (33, 70, 72, ("auto", "simple", "fp6")),
+    (9, 1000, 1920, ("skinny",)),           # the fallback streaming kernel
+    (2048, 2304, 1024, ("auto", "mfma")),   # 72 tiles of 256 x 256, several per workgroup
+])
+def test_linear_with_epilogue(gpu, host_threads, m, n, k, kernels):
+    import torch
+
+    import int4linear_amd as lib
+
+    rng = np.random.default_rng(m + n + k)
+    x = helpers.normal_s4(1200 + m, m, k)
+    w = helpers.uniform_s4(1300 + n, n, k)
+    bias = rng.integers(-100000, 100000, size=n, dtype=np.int32)
+    rs = rng.uniform(0.01, 2.0, size=m).astype(np.float32)
+    cs = rng.uniform(0.01, 2.0, size=n).astype(np.float32)
+    prod = oracle.linear_ref(x, w, threads=host_threads)
+    want_s32 = oracle.epilogue(prod, bias)
+    want_f32 = oracle.epilogue(prod, bias, rs, cs, f32=True)
+    want_f32_nobias = oracle.epilogue(prod, None, rs, None, f32=True)
+    xd = helpers.to_device_bytes(helpers.pack_bytes(x))
+    wd = helpers.to_device_bytes(helpers.pack_bytes(w))
+    bd, rd, cd = (torch.from_numpy(a).to("cuda:0") for a in (bias, rs, cs))
+    for kern in kernels:
+        y = torch.full((m, n), 0x7BADBAD, dtype=torch.int32, device="cuda:0")
+        lib.linear_s32(xd, wd, bd, y, m, n, k, kernel=kern)
+        assert np.array_equal(y.cpu().numpy(), want_s32), f"s32 {kern}"
+        lib.linear_s32(xd, wd, None, y, m, n, k, kernel=kern)
+        assert np.array_equal(y.cpu().numpy(), prod), f"s32 without bias {kern}"
+        yf = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda:0")
+        lib.linear_f32(xd, wd, bd, rd, cd, yf, m, n, k, kernel=kern)
+        # bit-exact: one rounding in the cast, one per product, same order as the oracle
+        assert np.array_equal(yf.cpu().numpy().view(np.int32), want_f32.view(np.int32)), f"f32 {kern}"
+        lib.linear_f32(xd, wd, None, rd, None, yf, m, n, k, kernel=kern)
+        assert np.array_equal(yf.cpu().numpy().view(np.int32), want_f32_nobias.view(np.int32)), f"f32 row scale {kern}"
+
+
 # ---- configuration 5: adversarial ---------------------------------------------------------
 
 def test_cfg5_all_minus_eight_full_size(gpu):

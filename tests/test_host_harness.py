@@ -63,7 +63,7 @@ def test_benchmark_harness_reports_tops(gpu):
     r = subprocess.run([str(_binary("benchmark")), "--iters", "5", "--warmup", "2", "2048x2048x2048", "16x4096x4096"],
                        capture_output=True, text=True, timeout=300)
     assert r.returncode == 0, r.stdout + r.stderr
-    lines = re.findall(r"\[PERF\] (\d+)x(\d+)x(\d+) kernel=(\w+) median ([\d.]+) ms .* ([\d.]+) TOPS", r.stdout)
+    lines = re.findall(r"\[PERF\] (\d+)x(\d+)x(\d+) kernel=(\w+) epilogue=\w+ median ([\d.]+) ms .* ([\d.]+) TOPS", r.stdout)
     assert len(lines) == 2 and all(float(l[5]) > 0 for l in lines), r.stdout
 
 

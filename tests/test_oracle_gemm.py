@@ -101,3 +101,35 @@ def test_is_same():
     b[99] -= 1
     b[0] -= 1
     assert not oracle.is_same(a, b)
+
+
+# ---- the linear layer's epilogue ---------------------------------------------------------
+
+def test_epilogue_identities():
+    rng = np.random.default_rng(11)
+    y = rng.integers(-2**20, 2**20, size=(7, 13), dtype=np.int32)
+    assert np.array_equal(oracle.epilogue(y), y)                                  # no operands: unchanged
+    assert np.array_equal(oracle.epilogue(y, f32=True), y.astype(np.float32))    # scales of 1: the cast
+    ones_r, ones_c = np.ones(7, np.float32), np.ones(13, np.float32)
+    assert np.array_equal(oracle.epilogue(y, None, ones_r, ones_c, f32=True), y.astype(np.float32))
+
+
+def test_epilogue_against_numpy():
+    rng = np.random.default_rng(12)
+    m, n = 33, 50
+    y = rng.integers(-2**30, 2**30, size=(m, n), dtype=np.int32)
+    bias = rng.integers(-2**30, 2**30, size=n, dtype=np.int32)
+    # int32 bias add wraps like two's-complement hardware
+    want = (y.astype(np.int64) + bias.astype(np.int64)).astype(np.uint64).astype(np.uint32).view(np.int32) \
+        if False else ((y.astype(np.int64) + bias[None, :].astype(np.int64)) & 0xFFFFFFFF).astype(np.uint32).view(np.int32)
+    assert np.array_equal(oracle.epilogue(y, bias), want.reshape(m, n))
+    # scaled float output: cast rounds once, each product rounds once, row scale first
+    rs = rng.uniform(0.001, 3.0, size=m).astype(np.float32)
+    cs = rng.uniform(0.001, 3.0, size=n).astype(np.float32)
+    v = want.reshape(m, n).astype(np.float32)
+    wantf = (v * rs[:, None]) * cs[None, :]
+    got = oracle.epilogue(y, bias, rs, cs, f32=True)
+    assert got.dtype == np.float32 and np.array_equal(got.view(np.int32), wantf.view(np.int32))
+    # only one of the scales
+    assert np.array_equal(oracle.epilogue(y, None, rs, None, f32=True), y.astype(np.float32) * rs[:, None])
+    assert np.array_equal(oracle.epilogue(y, None, None, cs, f32=True), y.astype(np.float32) * cs[None, :])
