@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the packed-int4 linear-layer GEMM on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-decode] [--calibrate-copy]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-decode] [--no-extra] [--calibrate-copy]
 
 A step is one GEMM launch C[MxN] = A[MxK] * B[NxK]^T through the library's C ABI
 (int4linear_gemm_s4s4s32, asynchronous, on torch's current stream).  The workload is
@@ -16,7 +16,11 @@ One JSON line is printed.  Besides the whole-run figure it carries
                 kernel alone, on the launch stream) against the dense peak of the MFMA
                 type it issues,
   decode        the skinny-M weight-streaming kernel at M = 16 against HBM bandwidth,
-  cpu_baseline  the CPU oracle's loop nest timed on this host's cores on a row sample.
+  cpu_baseline  the CPU oracle's loop nest timed on this host's cores on a row sample,
+  int8_kernel   the same 8192^3 problem on the library's int8-MFMA kernel (the path that
+                needs no workspace), against the int8 MFMA dense peak,
+  vendor        hipBLASLt's int8 GEMM on the widened operands, timed by the C++ harness
+                tests/host/vendor_compare (which also checks both results agree bit for bit).
 """
 from __future__ import annotations
 
@@ -46,6 +50,24 @@ def packed_random(torch, rows: int, k: int, seed: int):
     g = torch.Generator(device="cuda")
     g.manual_seed(seed)
     return torch.randint(0, 256, (rows, k // 2), dtype=torch.uint8, device="cuda", generator=g)
+
+
+RAMP_MS = 60.0   # untimed load before the first timed leg, see ramp_clocks
+
+
+def ramp_clocks(torch, launch, sets, min_ms: float = RAMP_MS):
+    """Runs the workload untimed for min_ms.  After an idle period this device needs some
+    tens of milliseconds of load before it runs at its sustained speed (the first ~60 calls
+    of the 8192^3 GEMM take 360-400 us, later ones 315-330 us); a short warm-up of a few
+    steps would time that ramp instead of the kernel."""
+    t0 = time.perf_counter()
+    i = 0
+    while (time.perf_counter() - t0) * 1e3 < min_ms:
+        for _ in range(10):
+            launch(sets[i % len(sets)])
+            i += 1
+        torch.cuda.synchronize()
+    return i
 
 
 def time_launches(torch, launch, sets, steps: int, warmup: int):
@@ -93,6 +115,7 @@ def bench_gemm(torch, lib, steps: int, warmup: int):
         if st != 0:
             raise RuntimeError(f"int4linear_gemm_s4s4s32 failed with status {st}")
 
+    ramp_clocks(torch, launch, args)
     ev_ms, wall_ms = time_launches(torch, launch, args, steps, warmup)
 
     # The dominant kernel alone: the FP6 GEMM on operands converted beforehand.
@@ -147,6 +170,51 @@ def bench_decode(torch, lib, steps: int, warmup: int):
     return out
 
 
+def bench_int8_kernel(torch, lib, steps: int, warmup: int):
+    """8192^3 on the int8 MFMA kernel (kernel id 2), same rotation and timing as the headline."""
+    import ctypes
+
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    sets = []
+    for s in range(3):
+        sets.append((packed_random(torch, M, K, 1000 + s), packed_random(torch, N, K, 2000 + s),
+                     torch.empty((M, N), dtype=torch.int32, device="cuda")))
+    fn = raw_entry("int4linear_gemm_s4s4s32_ex")
+    args = [(a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K, 2, stream) for (a, b, c) in sets]
+
+    def launch(t):
+        st = fn(*t)
+        if st != 0:
+            raise RuntimeError(f"int4linear_gemm_s4s4s32_ex failed with status {st}")
+
+    ev_ms, _ = time_launches(torch, launch, args, steps, warmup)
+    tops = 2.0 * M * N * K / (ev_ms * 1e-3) / 1e12
+    return {"kernel": "mfma_gemm_kernel (v_mfma_i32_32x32x32_i8)", "kernel_ms": ev_ms, "TOPS": tops,
+            "frac_of_int8_peak": tops / INT8_MFMA_PEAK_TOPS}
+
+
+def vendor_line():
+    """hipBLASLt int8 at 8192^3 through the C++ harness; None when the harness is not built."""
+    import re
+    import subprocess
+
+    exe = ROOT / "tests" / "host" / "bin" / "vendor_compare"
+    if not exe.exists():
+        return None
+    try:
+        r = subprocess.run([str(exe), "--iters", "20", f"{M}x{N}x{K}"], capture_output=True, text=True, timeout=120)
+    except (OSError, subprocess.TimeoutExpired):
+        return None
+    m = re.search(r"hipBLASLt int8 ([\d.]+) ms ([\d.]+) TOPS \| int4linear \((\w+)\) ([\d.]+) ms ([\d.]+) TOPS \| "
+                  r"ratio ([\d.]+)x \| results (\w+)", r.stdout)
+    if not m:
+        return None
+    return {"library": "hipBLASLt int8 x int8 -> int32 on operands widened beforehand", "ms": float(m.group(1)),
+            "TOPS": float(m.group(2)), "int4linear_ms_same_protocol": float(m.group(4)),
+            "int4linear_TOPS_same_protocol": float(m.group(5)), "speedup": float(m.group(6)),
+            "results": m.group(7), "protocol": "per-launch events, 512 MiB cache-cleaning fill before each, median of 20"}
+
+
 def cpu_baseline(budget_s: float = 15.0):
     """The oracle's loop nest (oracle_linear_ref_mt) on a row sample of the 8192^3
     problem, all host threads the box grants us."""
@@ -167,9 +235,16 @@ def cpu_baseline(budget_s: float = 15.0):
     oracle.linear_ref(x, w, threads=threads)
     dt = time.perf_counter() - t0
     tops = 2.0 * rows * N * K / dt / 1e12
+    # the reference's own single-threaded loop nest on a smaller sample, for the per-core figure
+    rows1 = max(1, rows // (threads * 4))
+    t0 = time.perf_counter()
+    oracle.linear_ref(x[:rows1], w, threads=1)
+    dt1 = time.perf_counter() - t0
     return {"value": tops, "unit": "TOPS", "cores": threads, "kind": "port",
             "sample": f"{rows} of {M} rows of the 8192^3 problem (all {N} columns, full K), "
-                      f"{dt:.1f} s, oracle_linear_ref_mt with {threads} threads"}
+                      f"{dt:.1f} s, oracle_linear_ref_mt with {threads} threads",
+            "single_thread_TOPS": 2.0 * rows1 * N * K / dt1 / 1e12,
+            "single_thread_sample": f"{rows1} rows, {dt1:.1f} s, oracle_linear_ref"}
 
 
 def measured_traffic(kernel: str):
@@ -189,10 +264,11 @@ def measured_traffic(kernel: str):
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="skip the decode-shape leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the int8-kernel and vendor legs")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run four plain 1 GiB device copies first (a kernel of known traffic "
                          "to scale hardware byte counters by when profiling)")
@@ -244,6 +320,7 @@ def main() -> int:
         "dtype": "fp6-e2m3 operands, fp32 accumulate (exact integers)" if kernel == "fp6" else "int8",
         "data": "synthetic",
         "config": {"workload": "M=N=K=8192 s4*s4->s32 GEMM, uniform [-8,7], 3 rotating operand sets",
+                   "untimed_clock_ramp_ms": RAMP_MS,
                    "kernel": kernel, "M": M, "N": N, "K": K},
         "pct_of_int8_mfma_peak": 100.0 * tops_wall / INT8_MFMA_PEAK_TOPS,
         "roofline": {"bound": "mfma", "achieved": tops_kernel, "peak": peak,
@@ -260,6 +337,9 @@ def main() -> int:
         result["decode"] = dec
         big = [d for d in dec if d["shape"] != [16, 4096, 4096]]
         result["decode_GB/s_M16"] = sum(d["GB/s"] for d in big) / len(big)
+    if not args.no_extra:
+        result["int8_kernel"] = bench_int8_kernel(torch, lib, max(10, args.steps // 2), args.warmup)
+        result["vendor"] = vendor_line()
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline()
     print(json.dumps(result))

@@ -116,7 +116,7 @@ int pick_kernel(int m, int n, int k)
 
 // Runs the FP6 path on the device's internal workspace.  Calls on one stream are ordered
 // by the stream; a call on a different stream than the previous user first waits for
-// that user's GEMM to finish with the workspace.
+// everything the previous user's stream has been given so far, that GEMM included.
 int run_fp6(PerDevice *pd, const void *a, const void *b, void *c, int m, int n, int k,
             const Epilogue &ep, hipStream_t stream)
 {
@@ -147,14 +147,22 @@ int run_fp6(PerDevice *pd, const void *a, const void *b, void *c, int m, int n, 
         pd->ws_bytes = need;
     }
     if (pd->ws_used && pd->ws_stream != stream) {
-        e = hipStreamWaitEvent(stream, pd->ws_event, 0);
+        // The previous user ran on another stream: mark the point its stream has reached
+        // now (which is after that GEMM) and make this stream wait for it.  Recording here,
+        // only when the stream changes, keeps the common one-stream case free of events.
+        e = hipEventRecord(pd->ws_event, pd->ws_stream);
+        if (e == hipSuccess) {
+            e = hipStreamWaitEvent(stream, pd->ws_event, 0);
+        } else {
+            // The previous stream no longer exists (destroyed with work possibly still
+            // draining): wait for the whole device instead.
+            (void)hipGetLastError();
+            e = hipDeviceSynchronize();
+        }
         if (e != hipSuccess)
             return fail_hip(e);
     }
     e = launch_fp6(a, b, c, m, n, k, pd->ws, ep, pd->info, stream);
-    if (e != hipSuccess)
-        return fail_hip(e);
-    e = hipEventRecord(pd->ws_event, stream);
     if (e != hipSuccess)
         return fail_hip(e);
     pd->ws_stream = stream;

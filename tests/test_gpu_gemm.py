@@ -198,6 +198,32 @@ def test_linear_with_epilogue(gpu, host_threads, m, n, k, kernels):
         assert np.array_equal(yf.cpu().numpy().view(np.int32), want_f32_nobias.view(np.int32)), f"f32 row scale {kern}"
 
 
+def test_internal_workspace_shared_between_streams(gpu, host_threads):
+    """Calls that use the FP6 workspace from alternating streams, without any host
+    synchronisation in between: the library orders them itself."""
+    import torch
+
+    import int4linear_amd as lib
+
+    m, n, k = 512, 768, 1024
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    cases = []
+    for i in range(6):
+        x = helpers.uniform_s4(1400 + i, m, k)
+        w = helpers.uniform_s4(1500 + i, n, k)
+        cases.append((helpers.to_device_bytes(helpers.pack_bytes(x)), helpers.to_device_bytes(helpers.pack_bytes(w)),
+                      torch.full((m, n), -1, dtype=torch.int32, device="cuda:0"),
+                      oracle.linear_ref(x, w, threads=host_threads)))
+    torch.cuda.synchronize()
+    for rep in range(3):
+        for i, (xd, wd, yd, _) in enumerate(cases):
+            s = streams[i % 2]
+            lib.gemm_s4s4s32(xd, wd, yd, m, n, k, kernel="fp6", stream=s.cuda_stream)
+    torch.cuda.synchronize()
+    for i, (_, _, yd, want) in enumerate(cases):
+        assert np.array_equal(yd.cpu().numpy(), want), f"case {i}"
+
+
 # ---- configuration 5: adversarial ---------------------------------------------------------
 
 def test_cfg5_all_minus_eight_full_size(gpu):
