@@ -13,12 +13,14 @@
 // fetches, since the LDS position of a lane's data is fixed) keeps those reads free of
 // bank conflicts.
 //
-// A workgroup owns R groups of 16 consecutive rows of W (16*R columns of C) over the
-// whole of K.  Its S wavefronts split K into S slices of T tiles of 256 nibbles; a wave
-// issues every load of its slices before it waits for anything, multiplies, and the S
-// partial sums meet once in LDS.  Each wave fetches its own slice of X once and reuses it
-// for its R row groups, so larger R cuts the (L2-resident, but hot-line) X traffic.
-// No atomics, no workspace, and the result does not depend on timing.
+// The rows of W are split evenly over the CUs in steps of eight; a workgroup holds its
+// rows as R groups of 16 (the last one possibly half empty) over the whole of K.  Its S
+// wavefronts split K into S slices of T tiles of 256 nibbles; a wave issues every load
+// of its slices before it waits for anything, multiplies each row group as soon as it has
+// landed (loads complete in issue order, so that is a wait for a known number of younger
+// loads), and the S partial sums meet once in LDS.  Each wave fetches its own slice of X
+// once and reuses it for its R row groups, so larger R cuts the (L2-resident, but
+// hot-line) X traffic.  No atomics, no workspace, and the result does not depend on timing.
 #include "kernels.h"
 
 #include <utility>

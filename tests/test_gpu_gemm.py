@@ -224,6 +224,56 @@ def test_internal_workspace_shared_between_streams(gpu, host_threads):
         assert np.array_equal(yd.cpu().numpy(), want), f"case {i}"
 
 
+def test_hip_graph_capture_and_replay(gpu, host_threads):
+    """The allocation-free entry points are plain kernel launches, so a caller may capture them
+    in a HIP graph: caller-owned FP6 operands, the int8 kernel and the streaming kernel, replayed
+    three times with new operand contents and eager work in between."""
+    import torch
+
+    import int4linear_amd as lib
+
+    m, n, k = 320, 768, 512
+    ms, ns, ks = 16, 2048, 1024
+    xd = torch.zeros(m * k // 2, dtype=torch.uint8, device="cuda:0")
+    wd = torch.zeros(n * k // 2, dtype=torch.uint8, device="cuda:0")
+    xs = torch.zeros(ms * ks // 2, dtype=torch.uint8, device="cuda:0")
+    ws = torch.zeros(ns * ks // 2, dtype=torch.uint8, device="cuda:0")
+    xc = torch.zeros(lib.fp6_operand_bytes(m, k), dtype=torch.uint8, device="cuda:0")
+    wc = torch.zeros(lib.fp6_operand_bytes(n, k), dtype=torch.uint8, device="cuda:0")
+    y6 = torch.zeros((m, n), dtype=torch.int32, device="cuda:0")
+    y8 = torch.zeros((m, n), dtype=torch.int32, device="cuda:0")
+    ysk = torch.zeros((ms, ns), dtype=torch.int32, device="cuda:0")
+    lib.init()
+    torch.cuda.synchronize()
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        lib.fp6_convert(xd, xc, m, k)
+        lib.fp6_convert(wd, wc, n, k)
+        lib.gemm_fp6_converted(xc, wc, y6, m, n, k)
+        lib.gemm_s4s4s32(xd, wd, y8, m, n, k, kernel="mfma")
+        lib.gemm_s4s4s32(xs, ws, ysk, ms, ns, ks, kernel="skinny")
+
+    for rep in range(3):
+        x = helpers.uniform_s4(1600 + rep, m, k)
+        w = helpers.uniform_s4(1700 + rep, n, k)
+        x2 = helpers.normal_s4(1800 + rep, ms, ks)
+        w2 = helpers.uniform_s4(1900 + rep, ns, ks)
+        xd.copy_(helpers.to_device_bytes(helpers.pack_bytes(x)))
+        wd.copy_(helpers.to_device_bytes(helpers.pack_bytes(w)))
+        xs.copy_(helpers.to_device_bytes(helpers.pack_bytes(x2)))
+        ws.copy_(helpers.to_device_bytes(helpers.pack_bytes(w2)))
+        for y in (y6, y8, ysk):
+            y.fill_(-1)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        want = oracle.linear_ref(x, w, threads=host_threads)
+        assert np.array_equal(y6.cpu().numpy(), want), f"fp6, replay {rep}"
+        assert np.array_equal(y8.cpu().numpy(), want), f"int8, replay {rep}"
+        assert np.array_equal(ysk.cpu().numpy(), oracle.linear_ref(x2, w2, threads=host_threads)), f"skinny, replay {rep}"
+
+
 # ---- configuration 5: adversarial ---------------------------------------------------------
 
 def test_cfg5_all_minus_eight_full_size(gpu):

@@ -138,3 +138,13 @@ def test_host_packer_golden_words():
 def test_numpy_byte_packer_used_by_large_gpu_tests():
     v = helpers.uniform_s4(3, 33, 256)
     assert np.array_equal(helpers.pack_bytes(v), helpers.pack_words_as_bytes(v).reshape(33, -1))
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    root = Path(__file__).resolve().parent.parent
+    r = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode == 2 and "one GPU" in r.stderr and r.stdout.strip() == ""
