@@ -80,6 +80,11 @@ __device__ __forceinline__ void load16_untracked(v4i &dst, const void *gptr)
 }
 __device__ __forceinline__ void settle(v4i &v) { asm volatile("" : "+v"(v)); }
 
+// Largest workgroup a variant is launched with.  The register-X variant with many
+// fragments per lane (2 * T * FMX of 16 bytes) needs the 256-register budget of at most
+// eight waves per workgroup.
+constexpr int max_threads(int t, int fmx, bool xdma) { return (!xdma && t * fmx > 4) ? 512 : 1024; }
+
 // T tiles per wave, R row groups per workgroup, FMX 16-row groups of X (M <= 16*FMX).
 // XDMA: X tiles go through LDS like W; otherwise they are loaded into registers in
 // fragment layout (for K so long that X tiles do not fit in LDS next to the W staging).
@@ -91,7 +96,7 @@ __device__ __forceinline__ void settle(v4i &v) { asm volatile("" : "+v"(v)); }
 // the waves and stored as soon as it has landed, while the later groups are still in
 // flight, so only the last group's reduction is exposed after the last byte arrives.
 template <int T, int R, int FMX, bool XDMA>
-__global__ __launch_bounds__(1024) void skinny_kernel(const uint8_t *__restrict__ X,
+__global__ __launch_bounds__(max_threads(T, FMX, XDMA)) void skinny_kernel(const uint8_t *__restrict__ X,
                                                       const uint8_t *__restrict__ W,
                                                       int32_t *__restrict__ Y, int M, int N, int K,
                                                       int rows_blk, Epilogue ep)
@@ -355,64 +360,75 @@ struct Plan {
     int lds = 0;
 };
 
-// Largest S <= 16 with S * T == tiles for the smallest T <= 4.  Rows per workgroup: the
-// matrix split evenly over the CUs (in as few rounds as the LDS and accumulator limits
-// allow), rounded up to a multiple of 8; R is the number of 16-row groups that takes.
+// Which (T, R, FMX, XDMA) combinations exist as kernels.  The partial sums of a row group
+// (FMX KiB per wave) go where the wave's own tiles of that group were (T * 2 KiB), except
+// that with a single row group and X in LDS they may run on into the X tiles; the
+// register-X variant holds 2 * T * FMX 16-byte fragments per lane.
+constexpr bool variant_exists(int t, int r, int fmx, bool xdma)
+{
+    if (xdma)
+        return r == 1 || fmx <= 2 * t;
+    return fmx <= 2 * t && t * fmx <= 8;
+}
+
+// Splits K over the waves and picks the X path for r row groups per workgroup: the
+// smallest T <= 4 (most waves, S = tiles / T <= 16) whose staging fits in LDS, X through
+// LDS if possible.  Returns false if nothing fits.
+bool fit(int tiles, int fmx, int r, Plan &p)
+{
+    for (int t = 1; t <= 4; ++t) {
+        if (tiles % t != 0 || tiles / t > 16)
+            continue;
+        const int s = tiles / t;
+        for (int xd = 1; xd >= 0; --xd) {
+            const int lds = s * t * (r + (xd ? fmx : 0)) * kTileBytes;
+            if (variant_exists(t, r, fmx, xd != 0) && lds <= kMaxLds && s * 64 <= max_threads(t, fmx, xd != 0)) {
+                p.t = t;
+                p.s = s;
+                p.r = r;
+                p.fmx = fmx;
+                p.xdma = xd != 0;
+                p.lds = lds;
+                return true;
+            }
+        }
+    }
+    return false;
+}
+
+// Rows per workgroup: the matrix split evenly over the CUs, in as few rounds as the
+// largest feasible R allows, rounded up to a multiple of 8; R is then the number of
+// 16-row groups that takes (a power of two).
 bool make_plan(int m, int n, int k, int cu_count, Plan &p)
 {
     if (k % kTileK != 0)
         return false;
     const int tiles = k / kTileK;
-    p.fmx = (m + 15) / 16;
-    p.t = 0;
-    for (int t = 1; t <= 4; ++t)
-        if (tiles % t == 0 && tiles / t <= 16) {
-            p.t = t;
-            p.s = tiles / t;
-            break;
-        }
-    if (p.t == 0)
-        return false;
-    auto lds_for = [&](int r, bool xdma) { return p.s * p.t * (r + (xdma ? p.fmx : 0)) * kTileBytes; };
-    // largest R the limits allow (R in {1, 2, 4}, R * FMX <= 4 accumulator blocks)
+    const int fmx = (m + 15) / 16;
     int rmax = 0;
-    bool xdma = true;
-    for (int r = 4; r >= 1 && rmax == 0; r >>= 1) {
-        if (r * p.fmx > 4)
-            continue;
-        for (int xd = 1; xd >= 0; --xd) {
-            if (xd == 0 && (p.t != 4 || p.fmx > 2))
-                continue;  // the register-X variant exists for T == 4, M <= 32 only
-            if (lds_for(r, xd != 0) <= kMaxLds) {
-                rmax = r;
-                xdma = xd != 0;
-                break;
-            }
-        }
-    }
+    for (int r = 4; r >= 1 && rmax == 0; r >>= 1)
+        if (fit(tiles, fmx, r, p))
+            rmax = r;
     if (rmax == 0)
         return false;
     const long cus = cu_count > 0 ? cu_count : 1;
     const long rounds = (n + cus * 16 * rmax - 1) / (cus * 16 * rmax);
     const long per_block = (n + cus * rounds - 1) / (cus * rounds);
-    p.rows_blk = (int)((per_block + 7) / 8 * 8);
+    const int rows_blk = (int)((per_block + 7) / 8 * 8);
     int r = 1;
-    while (16 * r < p.rows_blk)
+    while (16 * r < rows_blk)
         r <<= 1;
-    p.r = r;  // <= rmax
-    // X through LDS whenever it fits for this R
-    p.xdma = lds_for(r, true) <= kMaxLds ? true : xdma;
-    if (!p.xdma && (p.t != 4 || p.fmx > 2))
+    if (!fit(tiles, fmx, r, p))  // r <= rmax, so this succeeds
         return false;
-    p.lds = lds_for(r, p.xdma);
-    return p.lds <= kMaxLds;
+    p.rows_blk = rows_blk;
+    return true;
 }
 
 template <int T, int R, int FMX, bool XDMA>
 hipError_t launch_plan(const Plan &p, const void *a, const void *b, void *c, int m, int n, int k,
                        const Epilogue &ep, hipStream_t stream)
 {
-    if constexpr (!XDMA && (FMX > 2 || R > 1)) {  // the register-X variant is only ever planned with R == 1
+    if constexpr (!variant_exists(T, R, FMX, XDMA)) {
         return p.s == 0 ? hipSuccess : hipErrorInvalidConfiguration;  // never planned
     } else {
     auto kern = skinny_kernel<T, R, FMX, XDMA>;
@@ -432,40 +448,56 @@ hipError_t dispatch_rf(const Plan &p, const void *a, const void *b, void *c, int
 #define I4L_CASE(R_, F_)                                                      \
     if (p.r == R_ && p.fmx == F_)                                             \
         return launch_plan<T, R_, F_, XDMA>(p, a, b, c, m, n, k, ep, stream);
-    I4L_CASE(4, 1)
-    I4L_CASE(2, 1)
-    I4L_CASE(1, 1)
-    I4L_CASE(2, 2)
-    I4L_CASE(1, 2)
-    I4L_CASE(1, 3)
-    I4L_CASE(1, 4)
+    I4L_CASE(4, 1) I4L_CASE(2, 1) I4L_CASE(1, 1)
+    I4L_CASE(4, 2) I4L_CASE(2, 2) I4L_CASE(1, 2)
+    I4L_CASE(4, 3) I4L_CASE(2, 3) I4L_CASE(1, 3)
+    I4L_CASE(4, 4) I4L_CASE(2, 4) I4L_CASE(1, 4)
 #undef I4L_CASE
     return hipErrorInvalidConfiguration;
 }
 
 }  // namespace
 
+namespace {
+
+template <bool XDMA>
+hipError_t dispatch_t(const Plan &p, const void *a, const void *b, void *c, int m, int n, int k,
+                      const Epilogue &ep, hipStream_t stream)
+{
+    switch (p.t) {
+    case 1:
+        return dispatch_rf<1, XDMA>(p, a, b, c, m, n, k, ep, stream);
+    case 2:
+        return dispatch_rf<2, XDMA>(p, a, b, c, m, n, k, ep, stream);
+    case 3:
+        return dispatch_rf<3, XDMA>(p, a, b, c, m, n, k, ep, stream);
+    case 4:
+        return dispatch_rf<4, XDMA>(p, a, b, c, m, n, k, ep, stream);
+    default:
+        return hipErrorInvalidConfiguration;
+    }
+}
+
+}  // namespace
+
 hipError_t skinny_init(const DeviceInfo &)
 {
-    // Every instantiation may use up to the full LDS of a CU.
-    static const int kRf[7][2] = {{4, 1}, {2, 1}, {1, 1}, {2, 2}, {1, 2}, {1, 3}, {1, 4}};
-    for (const auto &rf : kRf) {
-        Plan p;
-        p.s = 0;
-        p.r = rf[0];
-        p.fmx = rf[1];
-        hipError_t e = dispatch_rf<1, true>(p, nullptr, nullptr, nullptr, 0, 0, 0, Epilogue{}, nullptr);
-        if (e == hipSuccess)
-            e = dispatch_rf<2, true>(p, nullptr, nullptr, nullptr, 0, 0, 0, Epilogue{}, nullptr);
-        if (e == hipSuccess)
-            e = dispatch_rf<3, true>(p, nullptr, nullptr, nullptr, 0, 0, 0, Epilogue{}, nullptr);
-        if (e == hipSuccess)
-            e = dispatch_rf<4, true>(p, nullptr, nullptr, nullptr, 0, 0, 0, Epilogue{}, nullptr);
-        if (e == hipSuccess)
-            e = dispatch_rf<4, false>(p, nullptr, nullptr, nullptr, 0, 0, 0, Epilogue{}, nullptr);
-        if (e != hipSuccess)
-            return e;
-    }
+    // Every instantiation may use up to the full LDS of a CU (a plan with s == 0 is the
+    // set-up call of launch_plan).
+    for (int t = 1; t <= 4; ++t)
+        for (int r = 1; r <= 4; r <<= 1)
+            for (int fmx = 1; fmx <= 4; ++fmx) {
+                Plan p;
+                p.s = 0;
+                p.t = t;
+                p.r = r;
+                p.fmx = fmx;
+                hipError_t e = dispatch_t<true>(p, nullptr, nullptr, nullptr, 0, 0, 0, Epilogue{}, nullptr);
+                if (e == hipSuccess)
+                    e = dispatch_t<false>(p, nullptr, nullptr, nullptr, 0, 0, 0, Epilogue{}, nullptr);
+                if (e != hipSuccess)
+                    return e;
+            }
     return hipSuccess;
 }
 
@@ -478,20 +510,9 @@ hipError_t launch_skinny(const void *a, const void *b, void *c, int m, int n, in
                          const Epilogue &ep, const DeviceInfo &dev, hipStream_t stream)
 {
     Plan p;
-    if (make_plan(m, n, k, dev.cu_count, p)) {
-        if (!p.xdma)
-            return dispatch_rf<4, false>(p, a, b, c, m, n, k, ep, stream);
-        switch (p.t) {
-        case 1:
-            return dispatch_rf<1, true>(p, a, b, c, m, n, k, ep, stream);
-        case 2:
-            return dispatch_rf<2, true>(p, a, b, c, m, n, k, ep, stream);
-        case 3:
-            return dispatch_rf<3, true>(p, a, b, c, m, n, k, ep, stream);
-        default:
-            return dispatch_rf<4, true>(p, a, b, c, m, n, k, ep, stream);
-        }
-    }
+    if (make_plan(m, n, k, dev.cu_count, p))
+        return p.xdma ? dispatch_t<true>(p, a, b, c, m, n, k, ep, stream)
+                      : dispatch_t<false>(p, a, b, c, m, n, k, ep, stream);
     switch ((m + 15) / 16) {
     case 1:
         return launch_basic<1>(a, b, c, m, n, k, ep, stream);

@@ -103,6 +103,9 @@ def test_cfg4_decode(gpu, host_threads, m, n, k):
     (64, 4096, 8192), (16, 13200, 8192), (5, 6560, 12288), (32, 6556, 12288), (64, 1030, 16384),
     (16, 13112, 14336), (32, 6562, 14336), (40, 515, 14336), (9, 1000, 1920), (64, 200, 20480),
     (16, 14336, 4096 + 256), (3, 16, 4096),
+    # more than 16 rows of X with several row groups per workgroup (X in registers)
+    (64, 14336, 4096), (48, 14300, 4096), (32, 14336, 4096), (64, 4096, 2048), (33, 9000, 1024), (64, 14336, 512),
+    (40, 14336, 6144), (64, 3000, 8192),
 ])
 def test_skinny_plans(gpu, host_threads, m, n, k):
     x = helpers.normal_s4(500 + m + k, m, k)
