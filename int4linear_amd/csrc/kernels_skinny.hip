@@ -81,9 +81,12 @@ __device__ __forceinline__ void load16_untracked(v4i &dst, const void *gptr)
 __device__ __forceinline__ void settle(v4i &v) { asm volatile("" : "+v"(v)); }
 
 // Largest workgroup a variant is launched with.  The register-X variant with many
-// fragments per lane (2 * T * FMX of 16 bytes) needs the 256-register budget of at most
-// eight waves per workgroup.
-constexpr int max_threads(int t, int fmx, bool xdma) { return (!xdma && t * fmx > 4) ? 512 : 1024; }
+// fragments (2 * T * FMX of 16 bytes) and accumulators (R * FMX of 16 bytes) per lane
+// needs the 256-register budget of at most eight waves per workgroup.
+constexpr int max_threads(int t, int r, int fmx, bool xdma)
+{
+    return (!xdma && (t * fmx > 4 || (t * fmx == 4 && r * fmx >= 8))) ? 512 : 1024;
+}
 
 // T tiles per wave, R row groups per workgroup, FMX 16-row groups of X (M <= 16*FMX).
 // XDMA: X tiles go through LDS like W; otherwise they are loaded into registers in
@@ -96,10 +99,10 @@ constexpr int max_threads(int t, int fmx, bool xdma) { return (!xdma && t * fmx 
 // the waves and stored as soon as it has landed, while the later groups are still in
 // flight, so only the last group's reduction is exposed after the last byte arrives.
 template <int T, int R, int FMX, bool XDMA>
-__global__ __launch_bounds__(max_threads(T, FMX, XDMA)) void skinny_kernel(const uint8_t *__restrict__ X,
+__global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(const uint8_t *__restrict__ X,
                                                       const uint8_t *__restrict__ W,
                                                       int32_t *__restrict__ Y, int M, int N, int K,
-                                                      int rows_blk, Epilogue ep)
+                                                      int rows_blk, int passes, Epilogue ep)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int kWaveTiles = T * (R + (XDMA ? FMX : 0));
@@ -112,7 +115,8 @@ __global__ __launch_bounds__(max_threads(T, FMX, XDMA)) void skinny_kernel(const
     const int n_end = min(N, n0 + rows_blk);  // > n0
     const unsigned lds_base = (unsigned)(size_t)I4L_LDS(lds);
     const unsigned my_lds = lds_base + wave * kWaveTiles * kTileBytes;
-    const size_t kbyte0 = (size_t)wave * T * kTileRowBytes;  // this wave's slice of every row
+    const int himask = (int)0xF0F0F0F0u;
+    const uint8_t *mine = lds + wave * kWaveTiles * kTileBytes;
 
     // Fragment layout: lane l supplies row l%16 and, in step s of a tile, chunk
     // 4*s + l/16 (32 nibbles: even ones feed one MFMA, odd ones the next).
@@ -125,7 +129,21 @@ __global__ __launch_bounds__(max_threads(T, FMX, XDMA)) void skinny_kernel(const
     //      slot ^ swizzle.  Rows past the workgroup's (or the matrix's) end re-read the
     //      last valid row: every wave issues the same number of loads, which the waits
     //      below rely on, and nothing is read out of bounds.
+    //
+    // K longer than S * T tiles is covered in several passes: pass c takes the c-th run of
+    // S * T tiles, each wave refills its own LDS tiles (nobody else reads them, and its own
+    // reads of the previous pass have been consumed) and keeps accumulating.
     v4i xg[XDMA ? 1 : T][2][FMX];
+    v4i acc[R][FMX];
+#pragma unroll
+    for (int rg = 0; rg < R; ++rg)
+#pragma unroll
+        for (int f = 0; f < FMX; ++f)
+            acc[rg][f] = (v4i){0, 0, 0, 0};
+
+#pragma unroll 1
+    for (int pass = 0; pass < passes; ++pass) {
+    const size_t kbyte0 = (size_t)(pass * waves + wave) * T * kTileRowBytes;  // this wave's slice of every row
     {
         const int lrow = lane >> 3;
         int chunk[2];
@@ -168,17 +186,10 @@ __global__ __launch_bounds__(max_threads(T, FMX, XDMA)) void skinny_kernel(const
                 }
     }
 
-    const int himask = (int)0xF0F0F0F0u;
-    const uint8_t *mine = lds + wave * kWaveTiles * kTileBytes;
-
     // ---- one row group at a time
     [&]<int... RG>(std::integer_sequence<int, RG...>) {
         ([&] {
             constexpr int rg = RG;
-            v4i acc[FMX];
-#pragma unroll
-            for (int f = 0; f < FMX; ++f)
-                acc[f] = (v4i){0, 0, 0, 0};
             [&]<int... TT>(std::integer_sequence<int, TT...>) {
                 ([&] {
                     constexpr int t = TT;
@@ -203,21 +214,25 @@ __global__ __launch_bounds__(max_threads(T, FMX, XDMA)) void skinny_kernel(const
                         for (int f = 0; f < FMX; ++f) {
                             const v4i x = XDMA ? *(const v4i *)(mine + ((R + f) * T + t) * kTileBytes + off)
                                                : xg[XDMA ? 0 : t][s][f];
-                            acc[f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo, (x << 4) & himask, acc[f], 0, 0, 0);
-                            acc[f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi, x & himask, acc[f], 0, 0, 0);
+                            acc[rg][f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo, (x << 4) & himask, acc[rg][f], 0, 0, 0);
+                            acc[rg][f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi, x & himask, acc[rg][f], 0, 0, 0);
                         }
                     }
                 }(), ...);
             }(std::make_integer_sequence<int, T>{});
 
-            // The wave's partial sums of this group go where its own tiles of the group
-            // were (nobody else touches that area).
-            v4i *part = (v4i *)(mine + (rg * T) * kTileBytes);
+            // After the last pass the wave's partial sums of this group go where its own
+            // tiles of the group were (nobody else touches that area), while the later
+            // groups are still landing.
+            if (pass == passes - 1) {
+                v4i *part = (v4i *)(mine + (rg * T) * kTileBytes);
 #pragma unroll
-            for (int f = 0; f < FMX; ++f)
-                part[f * 64 + lane] = acc[f];
+                for (int f = 0; f < FMX; ++f)
+                    part[f * 64 + lane] = acc[rg][f];
+            }
         }(), ...);
     }(std::make_integer_sequence<int, R>{});
+    }  // passes
 
     // ---- the workgroup meets once; one wave per 16 x 16 block adds the S partials up
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's partials are in LDS
@@ -356,6 +371,7 @@ hipError_t launch_basic(const void *a, const void *b, void *c, int m, int n, int
 struct Plan {
     int t = 0, s = 0, r = 0, fmx = 0;
     int rows_blk = 0;  // rows of W per workgroup: a multiple of 8, <= 16 * r
+    int passes = 1;    // K = passes * s * t tiles
     bool xdma = true;
     int lds = 0;
 };
@@ -371,28 +387,31 @@ constexpr bool variant_exists(int t, int r, int fmx, bool xdma)
     return fmx <= 2 * t && t * fmx <= 8;
 }
 
-// Splits K over the waves and picks the X path for r row groups per workgroup: the
-// smallest T <= 4 (most waves, S = tiles / T <= 16) whose staging fits in LDS, X through
-// LDS if possible.  Returns false if nothing fits.
+// Splits K over the waves and picks the X path for r row groups per workgroup: a single
+// pass if any T <= 4 allows it (smallest T first: most waves, S = tiles / T <= 16), else
+// the fewest passes; X through LDS if possible.  Returns false if nothing fits.
 bool fit(int tiles, int fmx, int r, Plan &p)
 {
-    for (int t = 1; t <= 4; ++t) {
-        if (tiles % t != 0 || tiles / t > 16)
-            continue;
-        const int s = tiles / t;
-        for (int xd = 1; xd >= 0; --xd) {
-            const int lds = s * t * (r + (xd ? fmx : 0)) * kTileBytes;
-            if (variant_exists(t, r, fmx, xd != 0) && lds <= kMaxLds && s * 64 <= max_threads(t, fmx, xd != 0)) {
-                p.t = t;
-                p.s = s;
-                p.r = r;
-                p.fmx = fmx;
-                p.xdma = xd != 0;
-                p.lds = lds;
-                return true;
+    for (int passes = 1; passes <= 8; ++passes)
+        for (int t = 1; t <= 4; ++t) {
+            if (tiles % (t * passes) != 0 || tiles / (t * passes) > 16)
+                continue;
+            const int s = tiles / (t * passes);
+            for (int xd = 1; xd >= 0; --xd) {
+                const int lds = s * t * (r + (xd ? fmx : 0)) * kTileBytes;
+                if (variant_exists(t, r, fmx, xd != 0) && lds <= kMaxLds &&
+                    s * 64 <= max_threads(t, r, fmx, xd != 0)) {
+                    p.t = t;
+                    p.s = s;
+                    p.r = r;
+                    p.fmx = fmx;
+                    p.xdma = xd != 0;
+                    p.lds = lds;
+                    p.passes = passes;
+                    return true;
+                }
             }
         }
-    }
     return false;
 }
 
@@ -436,7 +455,7 @@ hipError_t launch_plan(const Plan &p, const void *a, const void *b, void *c, int
         return hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
     const unsigned grid = (unsigned)((n + p.rows_blk - 1) / p.rows_blk);
     kern<<<grid, p.s * 64, p.lds, stream>>>((const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k,
-                                            p.rows_blk, ep);
+                                            p.rows_blk, p.passes, ep);
     return hipGetLastError();
     }
 }

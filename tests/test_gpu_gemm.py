@@ -106,6 +106,8 @@ def test_cfg4_decode(gpu, host_threads, m, n, k):
     # more than 16 rows of X with several row groups per workgroup (X in registers)
     (64, 14336, 4096), (48, 14300, 4096), (32, 14336, 4096), (64, 4096, 2048), (33, 9000, 1024), (64, 14336, 512),
     (40, 14336, 6144), (64, 3000, 8192),
+    # K covered in several passes
+    (64, 4096, 14336), (32, 4100, 14336), (16, 14336, 14336), (64, 500, 20480), (8, 700, 32768), (48, 1000, 12288),
 ])
 def test_skinny_plans(gpu, host_threads, m, n, k):
     x = helpers.normal_s4(500 + m + k, m, k)
