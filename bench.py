@@ -42,6 +42,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 
 M = N = K = 8192
 DECODE_SHAPES = [(16, 4096, 4096), (16, 14336, 4096), (16, 4096, 14336)]
+DECODE_OTHER_M = [(m, n, k) for m in (1, 64) for (n, k) in ((4096, 4096), (14336, 4096), (4096, 14336))]
 
 
 def packed_random(torch, rows: int, k: int, seed: int):
@@ -141,13 +142,13 @@ def bench_gemm(torch, lib, steps: int, warmup: int):
     return ev_ms, wall_ms, kernel, kern_ms
 
 
-def bench_decode(torch, lib, steps: int, warmup: int):
+def bench_decode(torch, lib, steps: int, warmup: int, shapes=None):
     import ctypes
 
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     gemm = raw_entry("int4linear_gemm_s4s4s32")
     out = []
-    for (m, n, k) in DECODE_SHAPES:
+    for (m, n, k) in (shapes or DECODE_SHAPES):
         wbytes = n * k // 2
         nsets = max(4, (768 << 20) // wbytes + 1)   # rotate through > 768 MiB of weights
         x = packed_random(torch, m, k, 31)
@@ -337,6 +338,7 @@ def main() -> int:
         result["decode"] = dec
         big = [d for d in dec if d["shape"] != [16, 4096, 4096]]
         result["decode_GB/s_M16"] = sum(d["GB/s"] for d in big) / len(big)
+        result["decode_other_M"] = bench_decode(torch, lib, args.steps, args.warmup, DECODE_OTHER_M)
     if not args.no_extra:
         result["int8_kernel"] = bench_int8_kernel(torch, lib, max(10, args.steps // 2), args.warmup)
         result["vendor"] = vendor_line()

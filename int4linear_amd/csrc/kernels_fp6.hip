@@ -104,6 +104,9 @@ struct ConvertJob {
 constexpr int kConvK = 512;                          // k per converter workgroup
 constexpr int kConvFrags = kConvK / kFragK;          // 8 fragments out
 constexpr int kConvChunks = kConvK / 32;             // 16-byte input chunks per row
+// LDS stride of a fragment being assembled: 64 bytes more than its size, so that the eight
+// lanes of a wave that write the same lane slot of different fragments hit different banks.
+constexpr int kConvFragLds = kFragBytes + 64;
 
 // One workgroup converts 32 rows x 512 k of one operand: thread t reads the 16-byte chunks
 // t%8 and t%8 + 8 of row t/8 (eight neighbouring lanes fetch a whole 128-byte line), the
@@ -116,7 +119,7 @@ constexpr int kConvChunks = kConvK / 32;             // 16-byte input chunks per
 template <bool ALIGNED16>
 __global__ __launch_bounds__(256) void fp6_convert_kernel(ConvertJob ja, ConvertJob jb, int k, int k_pad)
 {
-    __shared__ __attribute__((aligned(16))) uint8_t out[kConvFrags * kFragBytes];
+    __shared__ __attribute__((aligned(16))) uint8_t out[kConvFrags * kConvFragLds];
     const bool second = (int)blockIdx.y >= ja.row_blocks;
     const ConvertJob job = second ? jb : ja;
     const int rb = second ? blockIdx.y - ja.row_blocks : blockIdx.y;
@@ -155,7 +158,7 @@ __global__ __launch_bounds__(256) void fp6_convert_kernel(ConvertJob ja, Convert
         const unsigned long long o2 = (q2 >> 32) | (q3 << 16);
         const int kc = c + 8 * h;
         const int lane = (kc & 1) * 32 + r;
-        uint8_t *frag = out + (kc >> 1) * kFragBytes;
+        uint8_t *frag = out + (kc >> 1) * kConvFragLds;
         *(v4i *)(frag + lane * 16) = (v4i){(int)o0, (int)(o0 >> 32), (int)o1, (int)(o1 >> 32)};
         *(v2i *)(frag + kFragLoBytes + lane * 8) = (v2i){(int)o2, (int)(o2 >> 32)};
     }
@@ -171,7 +174,7 @@ __global__ __launch_bounds__(256) void fp6_convert_kernel(ConvertJob ja, Convert
         const int f = i / kVecPerFrag, v = i % kVecPerFrag;
         const int kfrag = kfrag0 + f;
         uint8_t *dst = job.dst + frag_offset(tile, kfrag / kFragsK, kfrag % kFragsK, rf, stages);
-        *(v4i *)(dst + v * 16) = *(const v4i *)(out + f * kFragBytes + v * 16);
+        *(v4i *)(dst + v * 16) = *(const v4i *)(out + f * kConvFragLds + v * 16);
     }
 }
 
