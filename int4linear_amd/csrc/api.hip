@@ -416,7 +416,7 @@ int int4linear_last_hip_error(void) { return t_last_hip_error; }
 
 size_t int4linear_workspace_bytes(int m, int n, int k)
 {
-    if (m < 0 || n < 0 || k < 0 || !fp6_worthwhile(m, n, k) || skinny_supports(m, n, k))
+    if (m < 1 || n < 1 || k < 8 || (k % 8) != 0 || pick_kernel(m, n, k) != INT4LINEAR_KERNEL_FP6)
         return 0;
     return fp6_workspace_bytes(m, n, k);
 }

@@ -98,6 +98,9 @@ def test_workspace_accounting():
     assert lib.workspace_bytes(4000, 8192, 4096) == (4096 + 8192) * 4096 * 3 // 4
     assert lib.workspace_bytes(16, 4096, 4096) == 0      # skinny kernel: none
     assert lib.workspace_bytes(1024, 1024, 1024) == 0    # int8 kernel: none
+    # K % 128 != 0 runs on the FP6 kernel: rows padded to 256, K to 128
+    assert lib.workspace_bytes(1000, 3000, 4104) == (1024 + 3072) * 4224 * 3 // 4
+    assert lib.workspace_bytes(0, 3000, 4096) == 0 and lib.workspace_bytes(8192, 8192, 12) == 0
     lib.set_workspace_limit(0)
     try:
         assert lib.workspace_bytes(8192, 8192, 8192) == 0
