@@ -279,6 +279,45 @@ def test_hip_graph_capture_and_replay(gpu, host_threads):
         assert np.array_equal(ysk.cpu().numpy(), oracle.linear_ref(x2, w2, threads=host_threads)), f"skinny, replay {rep}"
 
 
+def _random_shapes(count, seed):
+    rng = np.random.default_rng(seed)
+    shapes = []
+    for _ in range(count):
+        m = int(rng.integers(1, 65)) if rng.random() < 0.5 else int(rng.integers(65, 700))
+        n = int(rng.integers(1, 6000))
+        r = rng.random()
+        if r < 0.4:
+            k = 256 * int(rng.integers(1, 40))
+        elif r < 0.7:
+            k = 128 * int(rng.integers(1, 80))
+        else:
+            k = 8 * int(rng.integers(1, 600))
+        shapes.append((m, n, k))
+    return shapes
+
+
+@pytest.mark.parametrize("seed", [1, 2, 3, 4])
+def test_random_shapes_against_the_scalar_kernel(gpu, seed):
+    """Forty random shapes per seed through the automatic dispatch, whole outputs compared on
+    the device with the scalar kernel (itself checked against the oracle above): exercises the
+    plan search of the streaming kernel, tile edges and K padding on shapes nobody picked."""
+    import torch
+
+    import int4linear_amd as lib
+
+    g = torch.Generator(device="cuda:0")
+    for (m, n, k) in _random_shapes(40, seed):
+        g.manual_seed(m * 1000003 + n * 101 + k)
+        x = torch.randint(0, 256, (m * k // 2,), dtype=torch.uint8, device="cuda:0", generator=g)
+        w = torch.randint(0, 256, (n * k // 2,), dtype=torch.uint8, device="cuda:0", generator=g)
+        got = torch.full((m, n), 0x5A5A5A5A, dtype=torch.int32, device="cuda:0")
+        ref = torch.full((m, n), -1, dtype=torch.int32, device="cuda:0")
+        lib.gemm_s4s4s32(x, w, got, m, n, k)
+        lib.gemm_s4s4s32(x, w, ref, m, n, k, kernel="simple")
+        torch.cuda.synchronize()
+        assert torch.equal(got, ref), f"shape {(m, n, k)} kernel {lib.kernel_for_shape(m, n, k)}"
+
+
 # ---- configuration 5: adversarial ---------------------------------------------------------
 
 def test_cfg5_all_minus_eight_full_size(gpu):
