@@ -83,12 +83,15 @@ int ensure_init(PerDevice **out)
 
 bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 
-// The FP6 path pays off once its 256 x 256 tiles can occupy a good part of the device
-// (its converter pass is a fixed cost of about (M + N) * K * 1.25 bytes of HBM traffic).
+// The FP6 path pays off once its 256 x 256 tiles can occupy a good part of the device and K
+// is long enough to amortise the converter pass (a fixed cost of about (M + N) * K * 1.25
+// bytes of HBM traffic).  Measured crossovers against the int8 kernel: 128 tiles at K = 4096
+// and 256 tiles at K = 1024 still favour int8; 144 tiles at K = 3072, 256 tiles at K = 2048
+// and 1024 tiles at any K favour FP6.
 bool fp6_worthwhile(int m, int n, int k)
 {
     const long tiles = (long)((m + 255) / 256) * ((n + 255) / 256);
-    return fp6_supports(m, n, k) && tiles >= 128 &&
+    return fp6_supports(m, n, k) && tiles >= 144 && (k >= 2048 || tiles >= 1024) &&
            fp6_workspace_bytes(m, n, k) <= g_workspace_limit.load();
 }
 
