@@ -318,7 +318,9 @@ def main() -> int:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "fp6-e2m3 operands, fp32 accumulate (exact integers)" if kernel == "fp6" else "int8",
+        "dtype": "fp6" if kernel == "fp6" else "int8",
+        "dtype_note": ("s4 operands re-encoded exactly as FP6 E2M3, fp32 accumulation of integers below 2^24: "
+                       "bit-identical to int32 arithmetic") if kernel == "fp6" else "s4 widened to int8, int32 accumulation",
         "data": "synthetic",
         "config": {"workload": "M=N=K=8192 s4*s4->s32 GEMM, uniform [-8,7], 3 rotating operand sets",
                    "untimed_clock_ramp_ms": RAMP_MS,
