@@ -229,6 +229,49 @@ def test_internal_workspace_shared_between_streams(gpu, host_threads):
         assert np.array_equal(yd.cpu().numpy(), want), f"case {i}"
 
 
+def test_concurrent_host_threads(gpu, host_threads):
+    """Four host threads, each with its own stream, mixing kernels that share the internal
+    workspace with kernels that do not: the library serialises what has to be serialised."""
+    import threading
+
+    import torch
+
+    import int4linear_amd as lib
+
+    shapes = [(512, 768, 1024, "fp6"), (16, 2048, 1024, "auto"), (300, 520, 512, "mfma"), (640, 512, 384, "fp6")]
+    cases = []
+    for i, (m, n, k, kern) in enumerate(shapes):
+        x = helpers.uniform_s4(2000 + i, m, k)
+        w = helpers.uniform_s4(2100 + i, n, k)
+        cases.append((m, n, k, kern, helpers.to_device_bytes(helpers.pack_bytes(x)),
+                      helpers.to_device_bytes(helpers.pack_bytes(w)),
+                      torch.full((m, n), -1, dtype=torch.int32, device="cuda:0"),
+                      oracle.linear_ref(x, w, threads=host_threads)))
+    torch.cuda.synchronize()
+    errors = []
+
+    def worker(case):
+        m, n, k, kern, xd, wd, yd, want = case
+        try:
+            torch.cuda.set_device(0)
+            stream = torch.cuda.Stream()
+            for _ in range(25):
+                lib.gemm_s4s4s32(xd, wd, yd, m, n, k, kernel=kern, stream=stream.cuda_stream)
+            stream.synchronize()
+            if not np.array_equal(yd.cpu().numpy(), want):
+                errors.append(f"mismatch {(m, n, k, kern)}")
+        except Exception as exc:  # surfaced in the main thread below
+            errors.append(repr(exc))
+
+    threads = [threading.Thread(target=worker, args=(c,)) for c in cases]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not errors, errors
+
+
 def test_hip_graph_capture_and_replay(gpu, host_threads):
     """The allocation-free entry points are plain kernel launches, so a caller may capture them
     in a HIP graph: caller-owned FP6 operands, the int8 kernel and the streaming kernel, replayed
