@@ -276,7 +276,7 @@ def main() -> int:
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only; run with --gpus 1 "
-              "(the path shards over N with no exchange step, see DESIGN.md)", file=sys.stderr)
+              "(the path would shard over the rows of W with no exchange step)", file=sys.stderr)
         return 2
 
     import torch
