@@ -14,10 +14,12 @@
  *      with the reference's signatures and blocking behaviour, implemented on top of 1.
  *
  * All pointers named *_d are device pointers owned by the caller.  The only device
- * memory the library itself allocates is one workspace per device for the FP6 kernel
- * (see int4linear_workspace_bytes): created on first need, grown when a larger problem
- * arrives, never larger than the workspace limit, freed by int4linear_release_workspace
- * or at process exit.  With the limit set to 0 no entry point allocates anything.
+ * memory the library itself allocates is one workspace per device (see
+ * int4linear_workspace_bytes), which holds the FP6 kernel's converted operands or the
+ * partial sums of the int8 kernel's split-K form: created on first need, grown when a
+ * larger problem arrives, never larger than the workspace limit, freed by
+ * int4linear_release_workspace or at process exit.  With the limit set to 0 no entry
+ * point allocates anything.
  */
 #ifndef INT4LINEAR_H
 #define INT4LINEAR_H
@@ -107,8 +109,9 @@ int int4linear_fp6_convert(const void *packed_d, void *converted_d, int rows, in
 int int4linear_gemm_fp6_converted(const void *a_conv_d, const void *b_conv_d, void *c_d,
                                   int m, int n, int k, void *stream);
 
-/* Bytes of internal workspace INT4LINEAR_KERNEL_AUTO would use for a shape (0 when the
- * chosen kernel needs none). */
+/* Bytes of internal workspace INT4LINEAR_KERNEL_AUTO would use for a shape on the current
+ * device (0 when the chosen kernel needs none, and for the split-K form before the
+ * device's first call). */
 size_t int4linear_workspace_bytes(int m, int n, int k);
 
 /* Upper bound for the internal workspace (default 1 GiB).  Shapes that would need more,

@@ -117,16 +117,14 @@ int pick_kernel(int m, int n, int k)
     return INT4LINEAR_KERNEL_SIMPLE;
 }
 
-// Runs the FP6 path on the device's internal workspace.  Calls on one stream are ordered
-// by the stream; a call on a different stream than the previous user first waits for
-// everything the previous user's stream has been given so far, that GEMM included.
-int run_fp6(PerDevice *pd, const void *a, const void *b, void *c, int m, int n, int k,
-            const Epilogue &ep, hipStream_t stream)
+// Hands out the device's internal workspace with at least `need` bytes for work about to be
+// enqueued on `stream` (the caller holds pd->ws_mutex until that work is enqueued).  Calls
+// on one stream are ordered by the stream; a call on a different stream than the previous
+// user first waits for everything the previous user's stream has been given so far.
+int acquire_workspace(PerDevice *pd, size_t need, hipStream_t stream, void **out)
 {
-    const size_t need = fp6_workspace_bytes(m, n, k);
     if (need > g_workspace_limit.load())
         return INT4LINEAR_ERR_UNSUPPORTED;
-    std::lock_guard<std::mutex> lock(pd->ws_mutex);
     hipError_t e;
     if (!pd->ws_event) {
         e = hipEventCreateWithFlags(&pd->ws_event, hipEventDisableTiming);
@@ -151,8 +149,9 @@ int run_fp6(PerDevice *pd, const void *a, const void *b, void *c, int m, int n, 
     }
     if (pd->ws_used && pd->ws_stream != stream) {
         // The previous user ran on another stream: mark the point its stream has reached
-        // now (which is after that GEMM) and make this stream wait for it.  Recording here,
-        // only when the stream changes, keeps the common one-stream case free of events.
+        // now (which is after that user's kernels) and make this stream wait for it.
+        // Recording here, only when the stream changes, keeps the common one-stream case
+        // free of events.
         e = hipEventRecord(pd->ws_event, pd->ws_stream);
         if (e == hipSuccess) {
             e = hipStreamWaitEvent(stream, pd->ws_event, 0);
@@ -165,12 +164,42 @@ int run_fp6(PerDevice *pd, const void *a, const void *b, void *c, int m, int n, 
         if (e != hipSuccess)
             return fail_hip(e);
     }
-    e = launch_fp6(a, b, c, m, n, k, pd->ws, ep, pd->info, stream);
-    if (e != hipSuccess)
-        return fail_hip(e);
     pd->ws_stream = stream;
     pd->ws_used = true;
+    *out = pd->ws;
     return INT4LINEAR_OK;
+}
+
+// The FP6 path on the internal workspace.
+int run_fp6(PerDevice *pd, const void *a, const void *b, void *c, int m, int n, int k,
+            const Epilogue &ep, hipStream_t stream)
+{
+    std::lock_guard<std::mutex> lock(pd->ws_mutex);
+    void *ws = nullptr;
+    const int st = acquire_workspace(pd, fp6_workspace_bytes(m, n, k), stream, &ws);
+    if (st != INT4LINEAR_OK)
+        return st;
+    const hipError_t e = launch_fp6(a, b, c, m, n, k, ws, ep, pd->info, stream);
+    return e == hipSuccess ? INT4LINEAR_OK : fail_hip(e);
+}
+
+// The int8 kernel under automatic dispatch: split over K when that helps and the workspace
+// for the partial sums can be had, otherwise the plain kernel.
+int run_mfma_auto(PerDevice *pd, const void *a, const void *b, void *c, int m, int n, int k,
+                  const Epilogue &ep, hipStream_t stream)
+{
+    const size_t need = mfma_workspace_bytes(m, n, k, pd->info);
+    hipError_t e;
+    if (need == 0) {
+        e = launch_mfma(a, b, c, m, n, k, ep, pd->info, stream);
+    } else {
+        std::lock_guard<std::mutex> lock(pd->ws_mutex);
+        void *ws = nullptr;
+        if (acquire_workspace(pd, need, stream, &ws) != INT4LINEAR_OK)
+            ws = nullptr;  // no workspace: the unsplit kernel
+        e = launch_mfma_splitk(a, b, c, m, n, k, ws, ep, pd->info, stream);
+    }
+    return e == hipSuccess ? INT4LINEAR_OK : fail_hip(e);
 }
 
 int gemm_impl(const void *a, const void *b, void *c, int m, int n, int k, int kernel,
@@ -227,6 +256,8 @@ int gemm_impl(const void *a, const void *b, void *c, int m, int n, int k, int ke
     case INT4LINEAR_KERNEL_MFMA:
         if (!mfma_supports(m, n, k))
             return INT4LINEAR_ERR_UNSUPPORTED;
+        if (automatic)
+            return run_mfma_auto(pd, a, b, c, m, n, k, ep, stream);
         e = launch_mfma(a, b, c, m, n, k, ep, pd->info, stream);
         break;
     case INT4LINEAR_KERNEL_MFMA_128:
@@ -419,9 +450,20 @@ int int4linear_last_hip_error(void) { return t_last_hip_error; }
 
 size_t int4linear_workspace_bytes(int m, int n, int k)
 {
-    if (m < 1 || n < 1 || k < 8 || (k % 8) != 0 || pick_kernel(m, n, k) != INT4LINEAR_KERNEL_FP6)
+    if (m < 1 || n < 1 || k < 8 || (k % 8) != 0)
         return 0;
-    return fp6_workspace_bytes(m, n, k);
+    const int kernel = pick_kernel(m, n, k);
+    if (kernel == INT4LINEAR_KERNEL_FP6)
+        return fp6_workspace_bytes(m, n, k);
+    if (kernel == INT4LINEAR_KERNEL_MFMA) {
+        // the split-K form needs the device's CU count: 0 before the first call on a device
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices || g_devices[dev].info.cu_count == 0)
+            return 0;
+        const size_t need = mfma_workspace_bytes(m, n, k, g_devices[dev].info);
+        return need <= g_workspace_limit.load() ? need : 0;
+    }
+    return 0;
 }
 
 void int4linear_set_workspace_limit(size_t bytes) { g_workspace_limit.store(bytes); }

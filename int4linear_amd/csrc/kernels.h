@@ -46,6 +46,14 @@ hipError_t mfma_init(const DeviceInfo &dev);
 hipError_t launch_mfma(const void *a, const void *b, void *c, int m, int n, int k,
                        const Epilogue &ep, const DeviceInfo &dev, hipStream_t stream);
 
+// Split-K form for shapes with few tiles and long K: ksplit K-slices per 128 x 128 tile write
+// partial sums into `workspace` (mfma_workspace_bytes() bytes, 0 = the shape is not split),
+// a second kernel adds them up and applies the epilogue.  With a null workspace it is
+// launch_mfma.
+size_t mfma_workspace_bytes(int m, int n, int k, const DeviceInfo &dev);
+hipError_t launch_mfma_splitk(const void *a, const void *b, void *c, int m, int n, int k, void *workspace,
+                              const Epilogue &ep, const DeviceInfo &dev, hipStream_t stream);
+
 // The same kernel with the workgroup tile forced to 128 x 128 or 256 x 256 (`tile`).
 hipError_t launch_mfma_tile(const void *a, const void *b, void *c, int m, int n, int k, int tile,
                             const Epilogue &ep, const DeviceInfo &dev, hipStream_t stream);

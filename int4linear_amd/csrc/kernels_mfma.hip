@@ -130,7 +130,7 @@ __device__ __forceinline__ void tile_coords(int v, int total, int tiles_m, int t
 template <class C>
 __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
     const uint8_t *__restrict__ X, const uint8_t *__restrict__ W, int32_t *__restrict__ Y,
-    int M, int N, int K, int tiles_m, int tiles_n, Epilogue ep)
+    int M, int N, int K, int tiles_m, int tiles_n, int ksplit, Epilogue ep)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
@@ -139,11 +139,14 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
     const int wm = wave / C::WAVES_N;
     const int wn = wave % C::WAVES_N;
     const int rowbytes = K >> 1;
-    const int KT = K / kStageK;
-    const int total_tiles = tiles_m * tiles_n;
+    // With ksplit > 1 a work item is one K-slice of one tile: item v is slice v % ksplit of
+    // tile v / ksplit, covers KT stages, and stores its plain partial sums into slab
+    // v % ksplit of Y (M * N int32 each), which a second kernel adds up.
+    const int KT = K / kStageK / ksplit;
+    const int total_tiles = tiles_m * tiles_n * ksplit;  // work items
     const int nblk = gridDim.x;
     const int bid = blockIdx.x;
-    const bool ep_plain = !ep.bias && !ep.row_scale && !ep.col_scale && !ep.f32;
+    const bool ep_plain = ksplit > 1 || (!ep.bias && !ep.row_scale && !ep.col_scale && !ep.f32);
     if (bid >= total_tiles)
         return;
     const int my_tiles = (total_tiles - bid + nblk - 1) / nblk;
@@ -160,7 +163,8 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
 
     auto ld_setup_tile = [&](int it) {
         int tm, tn;
-        tile_coords(bid + it * nblk, total_tiles, tiles_m, tiles_n, tm, tn);
+        const int item = bid + it * nblk;
+        tile_coords(item / ksplit, total_tiles / ksplit, tiles_m, tiles_n, tm, tn);
         const int m0 = tm * C::BM, n0 = tn * C::BN;
         const int row = opaque(ld_row);
 #pragma unroll
@@ -172,8 +176,9 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
             const int rc = r < lim ? r : lim;
             voff[c] = (unsigned)rc * (unsigned)rowbytes + (unsigned)ld_c * 16u;
         }
-        xptr = X + (size_t)m0 * rowbytes;
-        wptr = W + (size_t)n0 * rowbytes;
+        const size_t k_off = (size_t)(item % ksplit) * KT * kRowBytes;
+        xptr = X + (size_t)m0 * rowbytes + k_off;
+        wptr = W + (size_t)n0 * rowbytes + k_off;
     };
 
     // One stage = CH loads per wave (ld_chunk) followed by the cursor advance.
@@ -452,11 +457,12 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
         if (kk == KT) {
             // ---- store the tile
             int tm, tn;
-            tile_coords(bid + cur_it * nblk, total_tiles, tiles_m, tiles_n, tm, tn);
+            const int item = bid + cur_it * nblk;
+            tile_coords(item / ksplit, total_tiles / ksplit, tiles_m, tiles_n, tm, tn);
             const int m0 = tm * C::BM, n0 = tn * C::BN;
             const int rows_left = M - m0;  // > 0
             const int cols_left = N - n0;  // > 0
-            int32_t *ybase = Y + (size_t)m0 * N + n0;
+            int32_t *ybase = Y + (size_t)(item % ksplit) * ((size_t)M * N) + (size_t)m0 * N + n0;
             // Byte extent of this tile's slab of C, measured from ybase.
             const size_t slab_rows = rows_left < C::BM ? rows_left : C::BM;
             const size_t extent = ((slab_rows - 1) * (size_t)N + (size_t)(cols_left < C::BN ? cols_left : C::BN)) * 4u;
@@ -538,6 +544,23 @@ using CfgLarge = TileConfig<2, 4, 4, 2, 4, 1>;
 // whose 256 x 256 tile count would leave CUs idle.
 using CfgMedium = TileConfig<2, 2, 2, 2, 4, 2>;
 
+// Second kernel of the split-K path: Y[i][j] = epilogue(sum over the ksplit partial slabs).
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const int32_t *__restrict__ partial,
+                                                            int32_t *__restrict__ Y, size_t count, int ksplit,
+                                                            int N, Epilogue ep)
+{
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= count)
+        return;
+    int sum = 0;
+    for (int s = 0; s < ksplit; ++s)
+        sum += partial[(size_t)s * count + i];
+    const size_t row = i / (size_t)N;
+    const int col = (int)(i - row * (size_t)N);
+    Y[i] = epilogue_value(ep, sum, ep.bias ? ep.bias[col] : 0, ep.row_scale ? ep.row_scale[row] : 1.f,
+                          ep.col_scale ? ep.col_scale[col] : 1.f);
+}
+
 template <class C>
 hipError_t set_lds_limit()
 {
@@ -547,11 +570,11 @@ hipError_t set_lds_limit()
 
 template <class C>
 hipError_t launch_cfg(const void *a, const void *b, void *c, int m, int n, int k,
-                      const Epilogue &ep, const DeviceInfo &dev, hipStream_t stream)
+                      const Epilogue &ep, const DeviceInfo &dev, hipStream_t stream, int ksplit = 1)
 {
     const int tiles_m = (m + C::BM - 1) / C::BM;
     const int tiles_n = (n + C::BN - 1) / C::BN;
-    const long total = (long)tiles_m * tiles_n;
+    const long total = (long)tiles_m * tiles_n * ksplit;
     if (total > 0x7fffffffL)
         return hipErrorInvalidValue;
     long grid = (long)dev.cu_count * C::OCC;
@@ -561,7 +584,7 @@ hipError_t launch_cfg(const void *a, const void *b, void *c, int m, int n, int k
     if ((size_t)C::BM * (size_t)n * 4u > 0x40000000ull)
         return hipErrorInvalidValue;
     mfma_gemm_kernel<C><<<(unsigned)grid, C::THREADS, C::LDS_BYTES, stream>>>(
-        (const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k, tiles_m, tiles_n, ep);
+        (const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k, tiles_m, tiles_n, ksplit, ep);
     return hipGetLastError();
 }
 
@@ -592,6 +615,53 @@ hipError_t launch_mfma_tile(const void *a, const void *b, void *c, int m, int n,
     if (tile == 128)
         return launch_cfg<CfgMedium>(a, b, c, m, n, k, ep, dev, stream);
     return hipErrorInvalidValue;
+}
+
+// K-slices per tile for shapes whose 128 x 128 tiles would fill at most an eighth of the
+// device at K >= 4096, or at most half of it at K >= 8192 (measured: with more tiles or
+// shorter K the second pass over the partial sums costs more than the idle CUs): the largest divisor of the stage count
+// that keeps at least eight stages per slice, at most eight slices, and at most half a
+// work item per slot.
+int mfma_ksplit(int m, int n, int k, const DeviceInfo &dev)
+{
+    if (!mfma_supports(m, n, k))
+        return 1;
+    const long tiles = (long)((m + CfgMedium::BM - 1) / CfgMedium::BM) * ((n + CfgMedium::BN - 1) / CfgMedium::BN);
+    const long slots = (long)dev.cu_count * CfgMedium::OCC;
+    const int stages = k / kStageK;
+    const bool few_tiles = tiles * 8 <= slots && stages >= 32;
+    const bool long_k = tiles * 2 <= slots && stages >= 64;
+    if (!few_tiles && !long_k)
+        return 1;
+    long limit = slots / (2 * tiles);
+    if (limit > 8)
+        limit = 8;
+    int best = 1;
+    for (int d = 2; d <= limit; ++d)
+        if (stages % d == 0 && stages / d >= 8)
+            best = d;
+    return best;
+}
+
+size_t mfma_workspace_bytes(int m, int n, int k, const DeviceInfo &dev)
+{
+    const int d = mfma_ksplit(m, n, k, dev);
+    return d > 1 ? (size_t)d * (size_t)m * (size_t)n * 4u : 0;
+}
+
+hipError_t launch_mfma_splitk(const void *a, const void *b, void *c, int m, int n, int k, void *workspace,
+                              const Epilogue &ep, const DeviceInfo &dev, hipStream_t stream)
+{
+    const int d = mfma_ksplit(m, n, k, dev);
+    if (d <= 1 || !workspace)
+        return launch_mfma(a, b, c, m, n, k, ep, dev, stream);
+    hipError_t e = launch_cfg<CfgMedium>(a, b, workspace, m, n, k, Epilogue{}, dev, stream, d);
+    if (e != hipSuccess)
+        return e;
+    const size_t count = (size_t)m * (size_t)n;
+    splitk_reduce_kernel<<<(unsigned)((count + 255) / 256), 256, 0, stream>>>((const int32_t *)workspace, (int32_t *)c,
+                                                                              count, d, n, ep);
+    return hipGetLastError();
 }
 
 hipError_t launch_mfma(const void *a, const void *b, void *c, int m, int n, int k,

@@ -229,6 +229,45 @@ def test_internal_workspace_shared_between_streams(gpu, host_threads):
         assert np.array_equal(yd.cpu().numpy(), want), f"case {i}"
 
 
+@pytest.mark.parametrize("m, n, k", [(128, 4096, 14336), (128, 4096, 4096), (300, 520, 4096), (1024, 512, 8192),
+                                     (65, 1000, 4096), (200, 136, 16384)])
+def test_split_k_form_of_the_int8_kernel(gpu, host_threads, m, n, k):
+    """Few tiles and long K: automatic dispatch splits K over workgroups (partial sums in the
+    internal workspace, a second kernel adds them and applies the epilogue)."""
+    import torch
+
+    import int4linear_amd as lib
+
+    x = helpers.uniform_s4(2200 + m, m, k)
+    w = helpers.uniform_s4(2300 + n, n, k)
+    want = oracle.linear_ref(x, w, threads=host_threads)
+    xp, wp = helpers.pack_bytes(x), helpers.pack_bytes(w)
+    assert lib.kernel_for_shape(m, n, k) == "mfma"
+    lib.init()
+    assert lib.workspace_bytes(m, n, k) > 0 and lib.workspace_bytes(m, n, k) % (m * n * 4) == 0
+    assert np.array_equal(helpers.run_gemm(xp, wp, m, n, k, kernel="auto"), want)
+    # the epilogue moves into the second kernel
+    rng = np.random.default_rng(m + k)
+    bias = rng.integers(-1000, 1000, size=n, dtype=np.int32)
+    rs = rng.uniform(0.1, 2.0, size=m).astype(np.float32)
+    cs = rng.uniform(0.1, 2.0, size=n).astype(np.float32)
+    xd, wd = helpers.to_device_bytes(xp), helpers.to_device_bytes(wp)
+    bd, rd, cd = (torch.from_numpy(a).to("cuda:0") for a in (bias, rs, cs))
+    y = torch.full((m, n), -1, dtype=torch.int32, device="cuda:0")
+    lib.linear_s32(xd, wd, bd, y, m, n, k)
+    assert np.array_equal(y.cpu().numpy(), oracle.epilogue(want, bias))
+    yf = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda:0")
+    lib.linear_f32(xd, wd, bd, rd, cd, yf, m, n, k)
+    assert np.array_equal(yf.cpu().numpy().view(np.int32), oracle.epilogue(want, bias, rs, cs, f32=True).view(np.int32))
+    # without a workspace the same call runs unsplit
+    lib.set_workspace_limit(0)
+    try:
+        assert lib.workspace_bytes(m, n, k) == 0
+        assert np.array_equal(helpers.run_gemm(xp, wp, m, n, k, kernel="auto"), want)
+    finally:
+        lib.set_workspace_limit(1 << 30)
+
+
 def test_concurrent_host_threads(gpu, host_threads):
     """Four host threads, each with its own stream, mixing kernels that share the internal
     workspace with kernels that do not: the library serialises what has to be serialised."""
