@@ -251,7 +251,7 @@ def cpu_baseline(budget_s: float = 15.0):
 def measured_traffic(kernel: str):
     """HBM bytes per launch of the GEMM kernel as recorded from rocprofv3 counter runs
     (FETCH_SIZE and WRITE_SIZE, each scaled by a plain copy of known size), or None."""
-    f = ROOT / "profiles" / "bench_default_hbm_traffic.md"
+    f = ROOT / "profiles" / "fp6_gemm_8192_and_decode_hbm_traffic.md"
     if f.exists():
         for line in f.read_text().splitlines():
             if line.startswith(f"bytes_per_launch {kernel}_gemm_8192:"):
