@@ -13,6 +13,17 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (gfx950) device")
 
 
+def pytest_sessionstart(session):
+    """The tests load what has been built; only if no library is there do they build it (the
+    product itself never builds or falls back: int4linear_amd._lib.load raises)."""
+    from int4linear_amd import _lib
+
+    if not _lib.LIB_PATH.exists():
+        from int4linear_amd.build import build_library
+
+        build_library()
+
+
 @pytest.fixture(scope="session")
 def gpu():
     """Device handle for GPU tests; fails (not skips) if the HIP library is missing."""
