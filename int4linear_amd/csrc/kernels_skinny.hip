@@ -38,21 +38,37 @@ constexpr int kTileRowBytes = kTileK / 2;   // one 128-byte line per row
 constexpr int kTileBytes = 16 * kTileRowBytes;  // 16 rows: 2 KiB
 constexpr int kMaxLds = 160 * 1024;
 
-// 16 bytes per lane from a per-lane global address straight into LDS at lds_addr +
-// 16*lane.  NT marks the weight stream as read-once.
-template <bool NT>
-__device__ __forceinline__ void dma16(const void *gptr, unsigned lds_addr)
+// Loads address memory as a wave-uniform base (scalar registers) plus a per-lane 32-bit
+// byte offset plus the compile-time constant IMM (0 .. 4095): one vector register per
+// distinct lane pattern, whatever the number of loads made with it.
+//
+// 16 bytes per lane straight into LDS at lds_addr + 16*lane.  NT marks the weight stream
+// as read-once.  The hardware adds the instruction's constant to the LDS address as well
+// as to the memory address, so it is taken off the LDS base here.
+template <bool NT, int IMM>
+__device__ __forceinline__ void dma16(const void *base, unsigned lane_off, unsigned lds_addr)
 {
+    static_assert(IMM >= 0 && IMM < 4096, "13-bit signed immediate");
+    lds_addr -= IMM;
     if (NT)
-        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt"
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%3 nt"
                      :
-                     : "v"(gptr), "s"(lds_addr)
+                     : "v"(lane_off), "s"(base), "s"(lds_addr), "n"(IMM)
                      : "memory");
     else
-        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%3"
                      :
-                     : "v"(gptr), "s"(lds_addr)
+                     : "v"(lane_off), "s"(base), "s"(lds_addr), "n"(IMM)
                      : "memory");
+}
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>)
+template <int N, class F>
+__device__ __forceinline__ void static_for(F &&f)
+{
+    [&]<int... I>(std::integer_sequence<int, I...>) {
+        (f(std::integral_constant<int, I>{}), ...);
+    }(std::make_integer_sequence<int, N>{});
 }
 
 // LDS slot (16 bytes) of chunk c of tile row r: c ^ ((r >> 1) & 7).  Rows are 128 B apart,
@@ -74,11 +90,34 @@ __device__ __forceinline__ void wait_vm_imm()
 // 16 bytes per lane from global memory into registers, invisible to the compiler's own
 // wait-count bookkeeping (which would otherwise wait for the younger weight loads too).
 // The value is only valid after a wait_vm_imm that covers it and a settle().
-__device__ __forceinline__ void load16_untracked(v4i &dst, const void *gptr)
+template <int IMM>
+__device__ __forceinline__ void load16_untracked(v4i &dst, const void *base, unsigned lane_off)
 {
-    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(gptr) : "memory");
+    static_assert(IMM >= 0 && IMM < 4096, "13-bit signed immediate");
+    asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3" : "=v"(dst) : "v"(lane_off), "s"(base), "n"(IMM) : "memory");
 }
 __device__ __forceinline__ void settle(v4i &v) { asm volatile("" : "+v"(v)); }
+
+// Transposes a 4 x 4 arrangement of 16-byte values inside every quad of lanes: on return
+// r[t] of lane j (j = lane % 4) holds what r[j] of lane t of the same quad held.  Two
+// exchange steps (lane distance 2, then 1), each a quad permutation and a select.
+__device__ __forceinline__ void quad_transpose(v4i &r0, v4i &r1, v4i &r2, v4i &r3, int lane)
+{
+    const bool up2 = (lane & 2) != 0, up1 = (lane & 1) != 0;
+    auto exchange = [](v4i &a, v4i &b, bool upper, auto ctrl) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int fa = __builtin_amdgcn_mov_dpp(a[c], decltype(ctrl)::value, 0xF, 0xF, true);
+            const int fb = __builtin_amdgcn_mov_dpp(b[c], decltype(ctrl)::value, 0xF, 0xF, true);
+            a[c] = upper ? fb : a[c];
+            b[c] = upper ? b[c] : fa;
+        }
+    };
+    exchange(r0, r2, up2, std::integral_constant<int, 0x4E>{});  // quad_perm [2,3,0,1]
+    exchange(r1, r3, up2, std::integral_constant<int, 0x4E>{});
+    exchange(r0, r1, up1, std::integral_constant<int, 0xB1>{});  // quad_perm [1,0,3,2]
+    exchange(r2, r3, up1, std::integral_constant<int, 0xB1>{});
+}
 
 // Largest workgroup a variant is launched with.  The register-X variant with many
 // fragments (2 * T * FMX of 16 bytes) and accumulators (R * FMX of 16 bytes) per lane
@@ -133,6 +172,15 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
     // K longer than S * T tiles is covered in several passes: pass c takes the c-th run of
     // S * T tiles, each wave refills its own LDS tiles (nobody else reads them, and its own
     // reads of the previous pass have been consumed) and keeps accumulating.
+    // With X in registers and an even T the X loads are made in a form the memory pipeline
+    // takes at full rate (every quad of lanes reads 64 contiguous bytes of one row; the
+    // fragment form, in which neighbouring lanes read different rows, is served at less
+    // than a third of that) and turned into fragments by a transposition inside the quads.
+    // Over a pair of tiles (256 bytes of a row, chunks 0..15) register j of the pair then
+    // holds, for lane (fr, fg), chunk 4 * fg + j of row fr, and W is read from LDS to match.
+    constexpr bool kPairX = !XDMA && T % 2 == 0;
+    // Row groups of W issued before X: the weight stream starts at once, X follows.
+    constexpr int kGroupsBeforeX = (!XDMA && R > 1) ? 1 : 0;
     v4i xg[XDMA ? 1 : T][2][FMX];
     v4i acc[R][FMX];
 #pragma unroll
@@ -143,47 +191,73 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
 
 #pragma unroll 1
     for (int pass = 0; pass < passes; ++pass) {
-    const size_t kbyte0 = (size_t)(pass * waves + wave) * T * kTileRowBytes;  // this wave's slice of every row
     {
-        const int lrow = lane >> 3;
-        int chunk[2];
+    // Per-lane byte offsets of the loads, relative to the wave's slice of the workgroup's
+    // first row of W, or of row 0 of X.
+    // (Derived anew in every pass from a copy of the lane number that the compiler cannot
+    // see through: kept across the multiplication they would cost registers there.)
+    int lane_here = lane;
+    asm volatile("" : "+v"(lane_here));
+    const int lrow = lane_here >> 3;
+    unsigned w_off[R][2];
 #pragma unroll
-        for (int u = 0; u < 2; ++u)
-            chunk[u] = ((lane & 7) ^ slot_swizzle(lrow + 8 * u)) * 16;
-        if (XDMA) {
+    for (int rg = 0; rg < R; ++rg)
 #pragma unroll
-            for (int f = 0; f < FMX; ++f)
+        for (int u = 0; u < 2; ++u) {
+            const int wr = rg * 16 + lrow + 8 * u;
+            w_off[rg][u] = (unsigned)(wr < n_end - n0 ? wr : n_end - n0 - 1) * rowbytes +
+                           ((lane_here & 7) ^ slot_swizzle(lrow + 8 * u)) * 16;
+        }
+    // X: through LDS like W (two loads per tile); as fragments (row fr, 64 bytes of a tile
+    // per load); or in the paired form, where load j of a tile pair has quad q read row
+    // 4 * (q % 4) + j, bytes 64 * (q / 4) .. + 64 of the pair.
+    constexpr int kXPatterns = XDMA ? 2 : kPairX ? 4 : 1;
+    unsigned x_off[FMX][kXPatterns];
 #pragma unroll
-                for (int t = 0; t < T; ++t)
+    for (int f = 0; f < FMX; ++f)
 #pragma unroll
-                    for (int u = 0; u < 2; ++u) {
-                        const int xr = f * 16 + lrow + 8 * u;
-                        const uint8_t *src = X + (size_t)(xr < M ? xr : M - 1) * rowbytes + kbyte0 + chunk[u];
-                        dma16<false>(src + t * kTileRowBytes,
-                                     my_lds + ((R + f) * T + t) * kTileBytes + u * 1024);
-                    }
-        } else {
+        for (int j = 0; j < kXPatterns; ++j) {
+            const int q = lane_here >> 2;
+            const int xr = f * 16 + (XDMA ? lrow + 8 * j : kPairX ? 4 * (q & 3) + j : (lane_here & 15));
+            const int within = XDMA ? ((lane_here & 7) ^ slot_swizzle(lrow + 8 * j)) * 16
+                               : kPairX ? 64 * (q >> 2) + 16 * (lane_here & 3) : (lane_here >> 4) * 16;
+            x_off[f][j] = (unsigned)(xr < M ? xr : M - 1) * rowbytes + within;
+        }
+        const size_t kbyte0 = (size_t)(pass * waves + wave) * T * kTileRowBytes;  // this wave's slice of every row
+        const uint8_t *wbase = W + (size_t)n0 * rowbytes + kbyte0;
+        const uint8_t *xbase = X + kbyte0;
+        auto issue_w = [&](int rg) {
+            static_for<T>([&](auto t) {
 #pragma unroll
-            for (int f = 0; f < FMX; ++f) {
-                const int xr = f * 16 + fr;
-                const uint8_t *src = X + (size_t)(xr < M ? xr : M - 1) * rowbytes + kbyte0;
+                for (int u = 0; u < 2; ++u)
+                    dma16<true, t() * kTileRowBytes>(wbase, w_off[rg][u], my_lds + (rg * T + t()) * kTileBytes + u * 1024);
+            });
+        };
 #pragma unroll
-                for (int t = 0; t < T; ++t)
+        for (int rg = 0; rg < kGroupsBeforeX; ++rg)
+            issue_w(rg);
 #pragma unroll
-                    for (int s = 0; s < 2; ++s)
-                        load16_untracked(xg[t][s][f], src + t * kTileRowBytes + (4 * s + fg) * 16);
+        for (int f = 0; f < FMX; ++f) {
+            if constexpr (XDMA) {
+                static_for<T>([&](auto t) {
+#pragma unroll
+                    for (int u = 0; u < 2; ++u)
+                        dma16<false, t() * kTileRowBytes>(xbase, x_off[f][u],
+                                                          my_lds + ((R + f) * T + t()) * kTileBytes + u * 1024);
+                });
+            } else if constexpr (kPairX) {
+                static_for<2 * T>([&](auto j) {
+                    load16_untracked<(j() >> 2) * 2 * kTileRowBytes>(xg[XDMA ? 0 : j() >> 1][j() & 1][f], xbase, x_off[f][j() & 3]);
+                });
+            } else {
+                static_for<2 * T>([&](auto j) {  // tile j / 2, step j % 2
+                    load16_untracked<(j() >> 1) * kTileRowBytes + (j() & 1) * 64>(xg[XDMA ? 0 : j() >> 1][j() & 1][f], xbase, x_off[f][0]);
+                });
             }
         }
 #pragma unroll
-        for (int rg = 0; rg < R; ++rg)
-#pragma unroll
-            for (int t = 0; t < T; ++t)
-#pragma unroll
-                for (int u = 0; u < 2; ++u) {
-                    const int wr = n0 + rg * 16 + lrow + 8 * u;
-                    const uint8_t *src = W + (size_t)(wr < n_end ? wr : n_end - 1) * rowbytes + kbyte0 + chunk[u];
-                    dma16<true>(src + t * kTileRowBytes, my_lds + (rg * T + t) * kTileBytes + u * 1024);
-                }
+        for (int rg = kGroupsBeforeX; rg < R; ++rg)
+            issue_w(rg);
     }
 
     // ---- one row group at a time
@@ -193,31 +267,52 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
             [&]<int... TT>(std::integer_sequence<int, TT...>) {
                 ([&] {
                     constexpr int t = TT;
-                    // loads younger than tile (rg, t): the rest of this group and the later groups
-                    wait_vm_imm<((R - 1 - rg) * T + (T - 1 - t)) * 2>();
+                    // Loads younger than tile (rg, t): the rest of this group and the later
+                    // groups.  When X was issued after the first group(s) of W, those groups
+                    // also wait for X, i.e. for everything up to the first group after X.
+                    constexpr int kYounger = ((R - 1 - rg) * T + (T - 1 - t)) * 2;
+                    constexpr int kAfterX = (R - kGroupsBeforeX) * T * 2;
+                    wait_vm_imm<(rg < kGroupsBeforeX && kYounger > kAfterX) ? kAfterX : kYounger>();
                     if (!XDMA && rg == 0 && t == 0) {
+                        // X has landed: the fragments are formed group by group
 #pragma unroll
-                        for (int tt = 0; tt < (XDMA ? 1 : T); ++tt)
+                        for (int f = 0; f < FMX; ++f)
 #pragma unroll
-                            for (int s = 0; s < 2; ++s)
+                            for (int tp = 0; tp < (XDMA ? 1 : T) / (kPairX ? 2 : 1); ++tp) {
+                                constexpr int kTilesHere = kPairX ? 2 : 1;
 #pragma unroll
-                                for (int f = 0; f < FMX; ++f)
-                                    settle(xg[tt][s][f]);
+                                for (int h = 0; h < 2 * kTilesHere; ++h)
+                                    settle(xg[kTilesHere * tp + (h >> 1)][h & 1][f]);
+                                if constexpr (kPairX)
+                                    quad_transpose(xg[XDMA ? 0 : 2 * tp][0][f], xg[XDMA ? 0 : 2 * tp][1][f],
+                                                   xg[XDMA ? 0 : 2 * tp + 1][0][f], xg[XDMA ? 0 : 2 * tp + 1][1][f], lane);
+                            }
                     }
+                    // In the paired form a pair of tiles is multiplied when its second tile
+                    // has landed: step s of tile t is register j = 2 * (t % 2) + s of the pair,
+                    // whose chunk 4 * fg + j lies in tile fg / 2 of the pair.
+                    if (kPairX && t % 2 == 0)
+                        return;
 #pragma unroll
-                    for (int s = 0; s < 2; ++s) {
-                        const int off = fr * kTileRowBytes + (((4 * s + fg) ^ sw) * 16);
-                        const v4i w = *(const v4i *)(mine + (rg * T + t) * kTileBytes + off);
-                        const v4i wlo = (w << 4) & himask;
-                        const v4i whi = w & himask;
+                    for (int tq = (kPairX ? t - 1 : t); tq <= t; ++tq)
 #pragma unroll
-                        for (int f = 0; f < FMX; ++f) {
-                            const v4i x = XDMA ? *(const v4i *)(mine + ((R + f) * T + t) * kTileBytes + off)
-                                               : xg[XDMA ? 0 : t][s][f];
-                            acc[rg][f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo, (x << 4) & himask, acc[rg][f], 0, 0, 0);
-                            acc[rg][f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi, x & himask, acc[rg][f], 0, 0, 0);
+                        for (int s = 0; s < 2; ++s) {
+                            const int j = 2 * (tq & 1) + s;
+                            const int frag = fr * kTileRowBytes + (((4 * s + fg) ^ sw) * 16);
+                            const int off = kPairX ? (rg * T + (t - 1) + (fg >> 1)) * kTileBytes + fr * kTileRowBytes +
+                                                         (((4 * (fg & 1) + j) ^ sw) * 16)
+                                                   : (rg * T + t) * kTileBytes + frag;
+                            const v4i w = *(const v4i *)(mine + off);
+                            const v4i wlo = (w << 4) & himask;
+                            const v4i whi = w & himask;
+#pragma unroll
+                            for (int f = 0; f < FMX; ++f) {
+                                const v4i x = XDMA ? *(const v4i *)(mine + ((R + f) * T + t) * kTileBytes + frag)
+                                                   : xg[XDMA ? 0 : tq][s][f];
+                                acc[rg][f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo, (x << 4) & himask, acc[rg][f], 0, 0, 0);
+                                acc[rg][f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi, x & himask, acc[rg][f], 0, 0, 0);
+                            }
                         }
-                    }
                 }(), ...);
             }(std::make_integer_sequence<int, T>{});
 
@@ -225,10 +320,14 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
             // tiles of the group were (nobody else touches that area), while the later
             // groups are still landing.
             if (pass == passes - 1) {
-                v4i *part = (v4i *)(mine + (rg * T) * kTileBytes);
+                // Lane (fr, fg) holds Y[m = fr][n = 4 * fg ..+4) of the block; it goes to slot
+                // 16 * fg + (fr ^ 2 * fg), so that the reducing lane 4 * m + j can fetch
+                // (fr = m, fg = j) (neighbouring lanes then store neighbouring 16 bytes of
+                // a row of Y) and neither side runs into LDS bank conflicts.
+                v4i *part = (v4i *)(mine + (rg * T) * kTileBytes) + 16 * fg + (fr ^ (2 * fg));
 #pragma unroll
                 for (int f = 0; f < FMX; ++f)
-                    part[f * 64 + lane] = acc[rg][f];
+                    part[f * 64] = acc[rg][f];
             }
         }(), ...);
     }(std::make_integer_sequence<int, R>{});
@@ -238,26 +337,30 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's partials are in LDS
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-#pragma unroll
-    for (int b = 0; b < R * FMX; ++b) {
-        if (wave != b % waves)
-            continue;
+#pragma unroll 1
+    for (int b = wave; b < R * FMX; b += waves) {
         const int rg = b / FMX, f = b % FMX;
-        const v4i *p = (const v4i *)(lds + (rg * T) * kTileBytes) + f * 64 + lane;
-        // All sixteen reads are issued back to back (a loop over the runtime wave count
-        // would wait for each one); waves that do not exist re-read partial 0 and add zero.
-        v4i part[16];
+        const int om = lane >> 2, oj = lane & 3;  // this lane adds up and stores Y[om][4 * oj ..+4) of the block
+        const v4i *p = (const v4i *)(lds + (rg * T) * kTileBytes) + f * 64 + 16 * oj + (om ^ (2 * oj));
+        // All reads are issued back to back (a loop over the runtime wave count would wait
+        // for each one), eight or sixteen of them; waves that do not exist re-read partial 0
+        // and add zero.
+        auto add_up = [&](auto count) {
+            constexpr int kCount = decltype(count)::value;
+            v4i part[kCount];
 #pragma unroll
-        for (int wv = 0; wv < 16; ++wv)
-            part[wv] = p[(size_t)(wv < waves ? wv : 0) * (kWaveTiles * kTileBytes / 16)];
-        v4i sum = part[0];
+            for (int wv = 0; wv < kCount; ++wv)
+                part[wv] = p[(size_t)(wv < waves ? wv : 0) * (kWaveTiles * kTileBytes / 16)];
+            v4i total = part[0];
 #pragma unroll
-        for (int wv = 1; wv < 16; ++wv)
-            sum += wv < waves ? part[wv] : (v4i){0, 0, 0, 0};
+            for (int wv = 1; wv < kCount; ++wv)
+                total += wv < waves ? part[wv] : (v4i){0, 0, 0, 0};
+            return total;
+        };
+        v4i sum = waves <= 8 ? add_up(std::integral_constant<int, 8>{}) : add_up(std::integral_constant<int, 16>{});
         sum = sum >> 8;  // both operands carried a factor 16
-        // lane l: m = 16*f + l%16, n = n0 + 16*rg + 4*(l/16) + 0..3
-        const int m = f * 16 + fr;
-        const int n = n0 + rg * 16 + 4 * fg;
+        const int m = f * 16 + om;
+        const int n = n0 + rg * 16 + 4 * oj;
         if (m < M) {
             const float rs = ep.row_scale ? ep.row_scale[m] : 1.f;
 #pragma unroll
