@@ -47,12 +47,14 @@ typedef unsigned v4u __attribute__((ext_vector_type(4)));
 // 32-bit offset.  M0 carries the LDS address; one wait state separates its write from
 // the load that reads it.  The compiler does not count this load in its own vmcnt
 // bookkeeping, which only makes the waits it inserts for its own accesses stricter.
-__device__ __forceinline__ void dma16(const void *sbase, unsigned voff, unsigned lds_addr)
+// The LDS address is the sum of two scalars (a fixed place inside a stage buffer and the
+// buffer's offset in the ring), added on the way into M0.
+__device__ __forceinline__ void dma16(const void *sbase, unsigned voff, unsigned lds_place, unsigned lds_ring)
 {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+    asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  :
-                 : "v"(voff), "s"(sbase), "s"(lds_addr)
-                 : "memory");
+                 : "v"(voff), "s"(sbase), "s"(lds_place), "s"(lds_ring)
+                 : "memory", "scc");
 }
 
 // Hides a value's origin from the optimiser so that work derived from it stays where
@@ -181,24 +183,35 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
         wptr = W + (size_t)n0 * rowbytes + k_off;
     };
 
-    // One stage = CH loads per wave (ld_chunk) followed by the cursor advance.
-    auto ld_chunk = [&](int c) {
-        const int buf = issued % C::NSTAGE;
-        const unsigned dst = lds_base + buf * C::STAGE_BYTES;
+    // One stage = CH loads per wave (ld_chunk) followed by the cursor advance.  Chunk c of
+    // this wave always lands at the same place of a stage buffer; wr_ring is the offset of
+    // the buffer being filled (ring position issued % NSTAGE).
+    unsigned chunk_place[C::CH];
+#pragma unroll
+    for (int c = 0; c < C::CH; ++c) {
         const bool is_x = c < C::X_CH;
         const int ci = (is_x ? c : c - C::X_CH) * C::NWAVES + wave;
-        dma16(is_x ? xptr : wptr, voff[c], dst + (is_x ? 0 : C::BM * kRowBytes) + ci * kChunkBytes);
+        chunk_place[c] = lds_base + (is_x ? 0 : C::BM * kRowBytes) + ci * kChunkBytes;
+    }
+    unsigned wr_ring = 0;
+    auto ld_chunk = [&](int c) {
+        dma16(c < C::X_CH ? xptr : wptr, voff[c], chunk_place[c], wr_ring);
     };
+    // Past the last stage the cursor stays where it is: the loads go on, as refills of
+    // buffers already consumed with data nobody reads, so that every iteration of the
+    // stage loop issues the same loads and the wait counts are constants.
     auto ld_advance = [&]() {
         ++issued;
-        ++ld_k;
-        xptr += kRowBytes;
-        wptr += kRowBytes;
-        if (ld_k == KT) {
-            ld_k = 0;
-            ++ld_it;
-            if (ld_it < my_tiles)
+        wr_ring = wr_ring + C::STAGE_BYTES == C::LDS_BYTES ? 0u : wr_ring + C::STAGE_BYTES;
+        if (issued < total_stages) {
+            ++ld_k;
+            xptr += kRowBytes;
+            wptr += kRowBytes;
+            if (ld_k == KT) {
+                ld_k = 0;
+                ++ld_it;
                 ld_setup_tile(ld_it);
+            }
         }
     };
     auto ld_issue = [&]() {
@@ -211,8 +224,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
     ld_setup_tile(0);
 #pragma unroll 1
     for (int s = 0; s < C::NSTAGE - 1; ++s)
-        if (issued < total_stages)
-            ld_issue();
+        ld_issue();
 
     // ---- math side -------------------------------------------------------------------
     // Lane l of a 32x32x32 MFMA supplies row l%32 and 16 of the 32 k values of both
@@ -253,8 +265,8 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
     constexpr int kReadParts = 3;
     constexpr int kXPerPart = C::FM / (kReadParts - 1);
     static_assert(kXPerPart * (kReadParts - 1) == C::FM, "X fragments must split evenly");
-    auto read_part = [&](int st, int h, int part, v4i (&w)[C::FN], v4i (&x)[C::FM]) {
-        const uint8_t *stage = lds + (st % C::NSTAGE) * C::STAGE_BYTES;
+    auto read_part = [&](unsigned ring, int h, int part, v4i (&w)[C::FN], v4i (&x)[C::FM]) {
+        const uint8_t *stage = lds + ring;  // the stage's buffer
         if (part == 0) {
 #pragma unroll
             for (int i = 0; i < C::FN; ++i)
@@ -266,11 +278,12 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
         }
     };
 
-    // Op k (0..11) of widening one packed fragment: per dword d = k/3 a shift, its mask
-    // (even-k nibbles) and the mask of the unshifted word (odd-k nibbles).
+    // Op k (0..11) of widening one packed fragment: the four shifts first, then the masks of
+    // the shifted words (even-k nibbles), then the masks of the unshifted words (odd-k
+    // nibbles), so that no op directly follows the one it depends on.
     auto widen_op = [&](int k, const v4i &p, v4i &lo, v4i &hi) {
-        const int d = k / 3;
-        switch (k % 3) {
+        const int d = k % 4;
+        switch (k / 4) {
         case 0:
             lo[d] = p[d] << 4;
             break;
@@ -339,16 +352,13 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
     };
 
     // Stage 0 must have landed before the first read.
-    if (issued >= C::NSTAGE - 1)
-        __builtin_amdgcn_s_waitcnt(I4L_VMCNT((C::NSTAGE - 2) * C::CH));
-    else
-        __builtin_amdgcn_s_waitcnt(I4L_VMCNT(0));
+    __builtin_amdgcn_s_waitcnt(I4L_VMCNT((C::NSTAGE - 2) * C::CH));
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     // Pipeline fill: unit (0, 0) read, its W and its X fragment 0 widened.
 #pragma unroll
     for (int part = 0; part < kReadParts; ++part)
-        read_part(0, 0, part, pk_w[0], pk_x[0]);
+        read_part(0u, 0, part, pk_w[0], pk_x[0]);
 #pragma unroll
     for (int i = 0; i < C::FN; ++i)
 #pragma unroll
@@ -378,23 +388,24 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
     static_assert(C::CH % 2 == 0 && kDmaStride >= 1 && kDmaStride * C::CH == kPositions,
                   "load spreading needs CH places per half");
     const int wave_par = wave & 1;
-    bool loading = false;  // a stage's loads are partly issued
-    // Housekeeping common to both halves at position (j, slot): `read_st`/`read_h` name the
-    // unit whose fragments are read, `half_pos` is 0 in the second half of an iteration.
-    auto spread = [&](auto j_tag, auto slot_tag, int read_st, int read_h, int half_pos) {
+    // Housekeeping common to both halves at position (j, slot): `read_ring`/`read_h` name the
+    // unit whose fragments are read, `half_pos` is 0 in the second half of an iteration,
+    // `do_load` is false only in the first half of the very first iteration (nothing begun).
+    auto spread = [&](auto j_tag, auto slot_tag, unsigned read_ring, int read_h, int half_pos, bool do_load) {
         constexpr int pos = decltype(j_tag)::value * kSlots + decltype(slot_tag)::value;
 #pragma unroll
         for (int part = 0; part < kReadParts; ++part)
             if (pos == part * kPositions / kReadParts + 1)
-                read_part(read_st, read_h, part, pk_w[read_h], pk_x[read_h]);
+                read_part(read_ring, read_h, part, pk_w[read_h], pk_x[read_h]);
         constexpr int off = kDmaStride / 2;
         if constexpr (pos >= off && (pos - off) % kDmaStride == 0) {
             constexpr int idx = (pos - off) / kDmaStride;  // 0 .. CH-1
-            if (loading && wave_par == idx % 2)
+            if (do_load && wave_par == idx % 2)
                 ld_chunk(half_pos * (C::CH / 2) + idx / 2);
         }
     };
 
+    unsigned rd_cur = 0, rd_next = C::STAGE_BYTES;  // ring offsets of stages gs and gs+1
 #pragma unroll 1
     for (int gs = 0; gs < total_stages; ++gs) {
         if (kk == 0) {
@@ -409,49 +420,45 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
 
         // ---- first half: reads the second half of this stage, finishes the loads begun
         //      in the previous iteration
+        const bool begun = gs > 0;
         unit(std::integral_constant<int, 0>{}, [&](auto j_tag, auto slot_tag) {
             constexpr int j = decltype(j_tag)::value;
             constexpr int slot = decltype(slot_tag)::value;
-            spread(j_tag, slot_tag, gs, 1, 1);
+            spread(j_tag, slot_tag, rd_cur, 1, 1, begun);
             if constexpr (slot == kSlots - 1 && j == C::FM - 1) {
-                if (loading) {
+                if (begun)
                     ld_advance();
-                    loading = false;
-                }
             }
         });
 
         // ---- second half: makes stage gs+1 readable, reads its first half, begins the
-        //      loads of stage gs+3 into the buffer of stage gs-1
+        //      loads of stage gs+NSTAGE-1 into the buffer of stage gs-1
         unit(std::integral_constant<int, 1>{}, [&](auto j_tag, auto slot_tag) {
             constexpr int j = decltype(j_tag)::value;
             constexpr int slot = decltype(slot_tag)::value;
             if constexpr (slot == 0 && j == 0) {
                 // This wave's loads of stage gs+1 must have landed, then every wave's.
-                // Outstanding VMEM ops complete in order; normally one younger stage is in
-                // flight behind them, and in the first stage after a tile end the C stores
-                // of that tile sit behind them as well.  (One stage later the loads waited
-                // for were themselves issued after those stores, so the stores must be done.)
-                const int ahead = issued - 2 - gs;  // stages issued after stage gs+1
-                if (ahead >= 1) {
-                    if (cur_it > 0 && kk < 1) {
-                        constexpr int with_stores = C::CH + C::STORES;
-                        __builtin_amdgcn_s_waitcnt(I4L_VMCNT(with_stores < 63 ? with_stores : 63));
-                    } else {
-                        __builtin_amdgcn_s_waitcnt(I4L_VMCNT(C::CH));
-                    }
-                } else {
-                    __builtin_amdgcn_s_waitcnt(I4L_VMCNT(0));
-                }
+                // Outstanding VMEM ops complete in order; NSTAGE - 3 younger stages are in
+                // flight behind them, and the C stores of a finished tile as well while the
+                // stage waited for was issued wholly before those stores, i.e. for the first
+                // NSTAGE - 3 stages of the next tile (after that the loads waited for were
+                // themselves issued after the stores).  The counter holds at most 63: a larger
+                // allowance becomes 63, which only waits longer.
+                constexpr int plain = (C::NSTAGE - 3) * C::CH, with_stores = plain + C::STORES;
+                if (cur_it > 0 && kk < C::NSTAGE - 3)
+                    __builtin_amdgcn_s_waitcnt(I4L_VMCNT(with_stores < 63 ? with_stores : 63));
+                else
+                    __builtin_amdgcn_s_waitcnt(I4L_VMCNT(plain < 63 ? plain : 63));
                 __builtin_amdgcn_s_barrier();
                 asm volatile("" ::: "memory");
                 // Every wave is past its reads of stage gs-1: that buffer may be refilled.
-                loading = issued < total_stages;
             }
             // (past the last stage the reads fetch a stale buffer whose contents never reach
             // a stored tile; unconditional reads keep the LDS wait counts exact)
-            spread(j_tag, slot_tag, gs + 1, 0, 0);
+            spread(j_tag, slot_tag, rd_next, 0, 0, true);
         });
+        rd_cur = rd_next;
+        rd_next = rd_next + C::STAGE_BYTES == C::LDS_BYTES ? 0u : rd_next + C::STAGE_BYTES;
 
         ++kk;
         if (kk == KT) {
@@ -535,6 +542,9 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
             ++cur_it;
         }
     }
+    // The refills issued past the last stage must have landed before the workgroup's LDS
+    // is handed to another one.
+    __builtin_amdgcn_s_waitcnt(I4L_VMCNT(0));
 }
 
 // 256 x 256 tile, eight wavefronts of 128 (m) x 64 (n), one workgroup per CU, two
