@@ -104,9 +104,20 @@ bool fp6_for_ragged_k(int m, int n, int k)
            fp6_workspace_bytes(m, n, k) <= g_workspace_limit.load();
 }
 
-int pick_kernel(int m, int n, int k)
+// What is known of the current device: all zero before the first call on it.
+DeviceInfo current_device_info()
 {
-    if (skinny_supports(m, n, k))
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+        return DeviceInfo{};
+    return g_devices[dev].info;
+}
+
+// `dev` is the device the call runs on (cu_count 0 if it has not been set up yet: shapes
+// whose choice depends on the CU count then get the choice that does not).
+int pick_kernel(int m, int n, int k, const DeviceInfo &dev)
+{
+    if (skinny_preferred(m, n, k, dev))
         return INT4LINEAR_KERNEL_SKINNY;
     if (fp6_worthwhile(m, n, k))
         return INT4LINEAR_KERNEL_FP6;
@@ -236,7 +247,7 @@ int gemm_impl(const void *a, const void *b, void *c, int m, int n, int k, int ke
 
     const bool automatic = kernel == INT4LINEAR_KERNEL_AUTO;
     if (automatic)
-        kernel = pick_kernel(m, n, k);
+        kernel = pick_kernel(m, n, k, pd->info);
     if (kernel == INT4LINEAR_KERNEL_FP6) {
         if (!fp6_supports(m, n, k))
             return INT4LINEAR_ERR_UNSUPPORTED;
@@ -412,7 +423,7 @@ const char *int4linear_kernel_for_shape(int m, int n, int k)
 {
     if (m < 0 || n < 0 || k < 0 || (k % 8) != 0)
         return "invalid";
-    switch (pick_kernel(m, n, k)) {
+    switch (pick_kernel(m, n, k, current_device_info())) {
     case INT4LINEAR_KERNEL_SKINNY:
         return "skinny";
     case INT4LINEAR_KERNEL_FP6:
@@ -452,15 +463,15 @@ size_t int4linear_workspace_bytes(int m, int n, int k)
 {
     if (m < 1 || n < 1 || k < 8 || (k % 8) != 0)
         return 0;
-    const int kernel = pick_kernel(m, n, k);
+    const DeviceInfo info = current_device_info();
+    const int kernel = pick_kernel(m, n, k, info);
     if (kernel == INT4LINEAR_KERNEL_FP6)
         return fp6_workspace_bytes(m, n, k);
     if (kernel == INT4LINEAR_KERNEL_MFMA) {
         // the split-K form needs the device's CU count: 0 before the first call on a device
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices || g_devices[dev].info.cu_count == 0)
+        if (info.cu_count == 0)
             return 0;
-        const size_t need = mfma_workspace_bytes(m, n, k, g_devices[dev].info);
+        const size_t need = mfma_workspace_bytes(m, n, k, info);
         return need <= g_workspace_limit.load() ? need : 0;
     }
     return 0;
@@ -510,11 +521,11 @@ int version_kernel(int version, int m, int n, int k)
         return INT4LINEAR_KERNEL_AUTO;
     case 20:
         if (fp6_supports(m, n, k) && fp6_workspace_bytes(m, n, k) <= g_workspace_limit.load() &&
-            !skinny_supports(m, n, k))
+            !skinny_preferred(m, n, k, current_device_info()))
             return INT4LINEAR_KERNEL_FP6;
         [[fallthrough]];
     case 11:
-        if (skinny_supports(m, n, k))
+        if (skinny_preferred(m, n, k, current_device_info()))
             return INT4LINEAR_KERNEL_SKINNY;
         [[fallthrough]];
     case 10:
@@ -531,6 +542,7 @@ int version_kernel(int version, int m, int n, int k)
 void launch_version(const char *name, int version, void *x, void *w, void *y, int m, int n, int k)
 {
     const bool valid = m >= 0 && n >= 0 && k >= 0 && (k % 8) == 0;
+    ensure_init(nullptr);  // the choice below may depend on the device; a failure is reported by the launch
     launch_blocking(name, x, w, y, m, n, k, valid ? version_kernel(version, m, n, k) : INT4LINEAR_KERNEL_AUTO);
 }
 

@@ -72,8 +72,11 @@ hipError_t launch_fp6_gemm(const void *a_conv, const void *b_conv, void *c, int 
 hipError_t launch_fp6(const void *a, const void *b, void *c, int m, int n, int k, void *workspace,
                       const Epilogue &ep, const DeviceInfo &dev, hipStream_t stream);
 
-// Weight-streaming kernel for skinny M.  Requires M <= 64, K % 128 == 0.
+// Weight-streaming kernel for skinny M.  K % 128 == 0; M <= 64, or more (in runs of 64
+// rows) when K splits into 128-byte tiles that fit the kernel's plans.  skinny_preferred:
+// the shapes for which the automatic dispatch uses it.
 bool skinny_supports(int m, int n, int k);
+bool skinny_preferred(int m, int n, int k, const DeviceInfo &dev);
 hipError_t skinny_init(const DeviceInfo &dev);
 hipError_t launch_skinny(const void *a, const void *b, void *c, int m, int n, int k,
                          const Epilogue &ep, const DeviceInfo &dev, hipStream_t stream);

@@ -138,10 +138,10 @@ constexpr int max_threads(int t, int r, int fmx, bool xdma)
 // the waves and stored as soon as it has landed, while the later groups are still in
 // flight, so only the last group's reduction is exposed after the last byte arrives.
 template <int T, int R, int FMX, bool XDMA>
-__global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(const uint8_t *__restrict__ X,
+__global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(const uint8_t *__restrict__ X_all,
                                                       const uint8_t *__restrict__ W,
-                                                      int32_t *__restrict__ Y, int M, int N, int K,
-                                                      int rows_blk, int passes, Epilogue ep)
+                                                      int32_t *__restrict__ Y_all, int M_all, int N, int K,
+                                                      int rows_blk, int passes, Epilogue ep_all)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int kWaveTiles = T * (R + (XDMA ? FMX : 0));
@@ -162,6 +162,18 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
     const int fr = lane & 15;
     const int fg = lane >> 4;
     const int sw = slot_swizzle(fr);
+
+    // More than 16 * FMX rows of X are taken in runs of that many, one after the other: the
+    // workgroup's rows of W are then streamed again, from the caches they were just pulled
+    // through.
+#pragma unroll 1
+    for (int m_first = 0; m_first < M_all; m_first += 16 * FMX) {
+    const uint8_t *X = X_all + (size_t)m_first * rowbytes;
+    int32_t *Y = Y_all + (size_t)m_first * N;
+    const int M = min(M_all - m_first, 16 * FMX);
+    Epilogue ep = ep_all;
+    if (ep.row_scale)
+        ep.row_scale += m_first;
 
     // ---- loads.  Lane p of a direct-to-LDS instruction lands at 16*p: tile row p/8 (+8
     //      for the second instruction of a tile), slot p%8, so it fetches chunk
@@ -380,6 +392,10 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
             }
         }
     }
+    // the partial sums have been read: the next run may refill the tiles
+    if (m_first + 16 * FMX < M_all)
+        __builtin_amdgcn_s_barrier();
+    }  // runs of rows of X
 }
 
 // ---- fallback for K that is a multiple of 128 but does not split into tiles: the
@@ -471,6 +487,8 @@ hipError_t launch_basic(const void *a, const void *b, void *c, int m, int n, int
     return hipGetLastError();
 }
 
+constexpr int kMaxRows = 1024;  // of X: runs of 64 rows, each a pass over the workgroup's rows of W
+
 struct Plan {
     int t = 0, s = 0, r = 0, fmx = 0;
     int rows_blk = 0;  // rows of W per workgroup: a multiple of 8, <= 16 * r
@@ -526,7 +544,7 @@ bool make_plan(int m, int n, int k, int cu_count, Plan &p)
     if (k % kTileK != 0)
         return false;
     const int tiles = k / kTileK;
-    const int fmx = (m + 15) / 16;
+    const int fmx = m > 64 ? 4 : (m + 15) / 16;
     int rmax = 0;
     for (int r = 4; r >= 1 && rmax == 0; r >>= 1)
         if (fit(tiles, fmx, r, p))
@@ -623,9 +641,32 @@ hipError_t skinny_init(const DeviceInfo &)
     return hipSuccess;
 }
 
+// More than 64 rows of X need the tiled kernel (which takes them in runs of 64); the
+// fallback does not loop.
 bool skinny_supports(int m, int n, int k)
 {
-    return m >= 1 && m <= 64 && n >= 1 && k >= 128 && k % 128 == 0 && k <= 131071 - 127;
+    if (!(m >= 1 && n >= 1 && k >= 128 && k % 128 == 0 && k <= 131071 - 127))
+        return false;
+    if (m <= 64)
+        return true;
+    Plan p;
+    return m <= kMaxRows && make_plan(m, n, k, 1, p);
+}
+
+// Where the kernel is the fastest one: up to 64 rows of X always; up to 128 when one
+// workgroup per CU covers W and K needs a single pass (W is then streamed twice, the
+// second time through the caches, which still beats 128 x 128 tiles that leave more
+// than half of the CUs idle).
+bool skinny_preferred(int m, int n, int k, const DeviceInfo &dev)
+{
+    if (!skinny_supports(m, n, k))
+        return false;
+    if (m <= 64)
+        return true;
+    Plan p;
+    if (m > 128 || dev.cu_count <= 0 || !make_plan(m, n, k, dev.cu_count, p))
+        return false;
+    return p.passes == 1 && (n + p.rows_blk - 1) / p.rows_blk <= dev.cu_count;
 }
 
 hipError_t launch_skinny(const void *a, const void *b, void *c, int m, int n, int k,
@@ -635,6 +676,8 @@ hipError_t launch_skinny(const void *a, const void *b, void *c, int m, int n, in
     if (make_plan(m, n, k, dev.cu_count, p))
         return p.xdma ? dispatch_t<true>(p, a, b, c, m, n, k, ep, stream)
                       : dispatch_t<false>(p, a, b, c, m, n, k, ep, stream);
+    if (m > 64)
+        return hipErrorInvalidConfiguration;  // skinny_supports() says no
     switch ((m + 15) / 16) {
     case 1:
         return launch_basic<1>(a, b, c, m, n, k, ep, stream);

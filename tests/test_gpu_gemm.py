@@ -108,6 +108,10 @@ def test_cfg4_decode(gpu, host_threads, m, n, k):
     (40, 14336, 6144), (64, 3000, 8192),
     # K covered in several passes
     (64, 4096, 14336), (32, 4100, 14336), (16, 14336, 14336), (64, 500, 20480), (8, 700, 32768), (48, 1000, 12288),
+    # more than 64 rows of X: runs of 64 inside the kernel (the automatic choice up to 128 rows when one
+    # workgroup per CU covers W in a single pass over K, a forced one beyond)
+    (65, 4096, 4096), (128, 14336, 4096), (100, 3000, 2048), (96, 14336, 512), (128, 600, 14336),
+    (200, 520, 1024), (130, 20000, 4096),
 ])
 def test_skinny_plans(gpu, host_threads, m, n, k):
     x = helpers.normal_s4(500 + m + k, m, k)
@@ -167,6 +171,7 @@ def test_ragged_k_runs_on_the_fp6_kernel(gpu, host_threads, m, n, k):
     (300, 520, 512, ("auto", "simple", "mfma128", "mfma256", "fp6")),
     (16, 1024, 1024, ("auto", "skinny", "mfma", "fp6")),
     (40, 515, 14336, ("skinny",)),
+    (100, 4100, 4096, ("auto", "skinny")),   # two runs of rows of X: the row scales move with them
     (33, 70, 72, ("auto", "simple", "fp6")),
     (9, 1000, 1920, ("skinny",)),           # the fallback streaming kernel
     (2048, 2304, 1024, ("auto", "mfma")),   # 72 tiles of 256 x 256, several per workgroup
@@ -229,8 +234,8 @@ def test_internal_workspace_shared_between_streams(gpu, host_threads):
         assert np.array_equal(yd.cpu().numpy(), want), f"case {i}"
 
 
-@pytest.mark.parametrize("m, n, k", [(128, 4096, 14336), (128, 4096, 4096), (300, 520, 4096), (1024, 512, 8192),
-                                     (65, 1000, 4096), (200, 136, 16384)])
+@pytest.mark.parametrize("m, n, k", [(128, 4096, 14336), (160, 4096, 4096), (300, 520, 4096), (1024, 512, 8192),
+                                     (140, 1000, 4096), (200, 136, 16384)])
 def test_split_k_form_of_the_int8_kernel(gpu, host_threads, m, n, k):
     """Few tiles and long K: automatic dispatch splits K over workgroups (partial sums in the
     internal workspace, a second kernel adds them and applies the epilogue)."""
@@ -471,7 +476,7 @@ def test_degenerate_sizes(gpu):
     with pytest.raises(lib.Int4LinearError):
         lib.gemm_s4s4s32(a, a, y, 8, 12, 64, kernel="mfma")   # K below one stage
     with pytest.raises(lib.Int4LinearError):
-        lib.gemm_s4s4s32(a, a, y, 65, 12, 128, kernel="skinny")  # M too large
+        lib.gemm_s4s4s32(a, a, y, 65, 12, 128, kernel="skinny")  # more than 64 rows need K in 128-byte tiles
 
 
 # ---- properties that hold at any size -------------------------------------------------------
