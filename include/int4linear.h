@@ -46,7 +46,8 @@ enum {
     INT4LINEAR_KERNEL_AUTO = 0,   /* shape-based dispatch (what the plain entry uses)    */
     INT4LINEAR_KERNEL_SIMPLE = 1, /* one thread per output, scalar nibble decode; any K%8==0 */
     INT4LINEAR_KERNEL_MFMA = 2,   /* LDS-pipelined v_mfma_i32_32x32x32_i8 kernel; K%128==0 */
-    INT4LINEAR_KERNEL_SKINNY = 3, /* weight-streaming kernel for M <= 64; K%128==0       */
+    INT4LINEAR_KERNEL_SKINNY = 3, /* weight-streaming kernel: M <= 64 and K%128==0, or more
+                                     rows (in runs of 64) when K splits into 128-byte tiles */
     INT4LINEAR_KERNEL_FP6 = 4,    /* operands converted to FP6 (E2M3) in a workspace, then
                                      v_mfma_scale_f32_32x32x64_f8f6f4; exact; any K%8==0
                                      below 2^18 (the converter pads K to 128 with zeros) */
@@ -146,7 +147,7 @@ int int4linear_device_cu_count(void);
  *   v1   int8 MFMA kernel, 128x128 workgroup tile
  *   v2   int8 MFMA kernel, 256x256 workgroup tile
  *   v10  int8 MFMA kernel, tile chosen from the grid size
- *   v11  v10 plus the weight-streaming kernel for M <= 64
+ *   v11  v10 plus the weight-streaming kernel for skinny M
  *   v20  v11 plus the FP6 kernel wherever it can run
  *   v21  the full automatic dispatch (what int4linear_gemm_s4s4s32 does)
  * A version whose kernel cannot take a shape falls back to the one before it, so every
