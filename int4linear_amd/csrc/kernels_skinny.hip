@@ -137,7 +137,7 @@ constexpr int max_threads(int t, int r, int fmx, bool xdma)
 // wait for a fixed number of younger loads.  Each row group is multiplied, reduced across
 // the waves and stored as soon as it has landed, while the later groups are still in
 // flight, so only the last group's reduction is exposed after the last byte arrives.
-template <int T, int R, int FMX, bool XDMA>
+template <int T, int R, int FMX, bool XDMA, bool RAGGED>
 __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(const uint8_t *__restrict__ X_all,
                                                       const uint8_t *__restrict__ W,
                                                       int32_t *__restrict__ Y_all, int M_all, int N, int K,
@@ -201,6 +201,7 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
         for (int f = 0; f < FMX; ++f)
             acc[rg][f] = (v4i){0, 0, 0, 0};
 
+    int skip = 0;
 #pragma unroll 1
     for (int pass = 0; pass < passes; ++pass) {
     {
@@ -235,7 +236,14 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
                                : kPairX ? 64 * (q >> 2) + 16 * (lane_here & 3) : (lane_here >> 4) * 16;
             x_off[f][j] = (unsigned)(xr < M ? xr : M - 1) * rowbytes + within;
         }
-        const size_t kbyte0 = (size_t)(pass * waves + wave) * T * kTileRowBytes;  // this wave's slice of every row
+        // This wave's slice of every row: T tiles from tile (pass * S + wave) * T on.  When
+        // K's tiles do not fill the last slices, a slice that would run past the end is
+        // moved back to end with the last tile, and its first `skip` tiles (someone else's,
+        // or all T of them) are loaded like the others but not multiplied.
+        const int first_tile = (pass * waves + wave) * T;
+        if (RAGGED)
+            skip = max(0, first_tile + T - K / kTileK);
+        const size_t kbyte0 = (size_t)(first_tile - skip) * kTileRowBytes;
         const uint8_t *wbase = W + (size_t)n0 * rowbytes + kbyte0;
         const uint8_t *xbase = X + kbyte0;
         auto issue_w = [&](int rg) {
@@ -309,12 +317,21 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
                     for (int tq = (kPairX ? t - 1 : t); tq <= t; ++tq)
 #pragma unroll
                         for (int s = 0; s < 2; ++s) {
+                            // Tiles before `skip` are not this wave's.  In the paired form every
+                            // register spans both tiles of the pair (lanes with fg < 2 hold the
+                            // first one): the pair is left out if its second tile is, and only
+                            // the first tile's lanes are blanked if just that one is.
+                            if (RAGGED && (kPairX ? t : tq) < skip)
+                                continue;
+                            const bool blank_first = RAGGED && kPairX && t - 1 < skip;
                             const int j = 2 * (tq & 1) + s;
                             const int frag = fr * kTileRowBytes + (((4 * s + fg) ^ sw) * 16);
                             const int off = kPairX ? (rg * T + (t - 1) + (fg >> 1)) * kTileBytes + fr * kTileRowBytes +
                                                          (((4 * (fg & 1) + j) ^ sw) * 16)
                                                    : (rg * T + t) * kTileBytes + frag;
-                            const v4i w = *(const v4i *)(mine + off);
+                            v4i w = *(const v4i *)(mine + off);
+                            if (blank_first && fg < 2)
+                                w = (v4i){0, 0, 0, 0};
                             const v4i wlo = (w << 4) & himask;
                             const v4i whi = w & himask;
 #pragma unroll
@@ -494,6 +511,7 @@ struct Plan {
     int rows_blk = 0;  // rows of W per workgroup: a multiple of 8, <= 16 * r
     int passes = 1;    // K = passes * s * t tiles
     bool xdma = true;
+    bool ragged = false;  // S * T * passes > K's tiles: the last slices are partly or wholly empty
     int lds = 0;
 };
 
@@ -510,14 +528,15 @@ constexpr bool variant_exists(int t, int r, int fmx, bool xdma)
 
 // Splits K over the waves and picks the X path for r row groups per workgroup: a single
 // pass if any T <= 4 allows it (smallest T first: most waves, S = tiles / T <= 16), else
-// the fewest passes; X through LDS if possible.  Returns false if nothing fits.
-bool fit(int tiles, int fmx, int r, Plan &p)
+// the fewest passes; X through LDS if possible.  `ragged` admits splits whose last slices
+// are partly or wholly empty (S * T * passes > tiles).  Returns false if nothing fits.
+bool fit(int tiles, int fmx, int r, bool ragged, Plan &p)
 {
     for (int passes = 1; passes <= 8; ++passes)
         for (int t = 1; t <= 4; ++t) {
-            if (tiles % (t * passes) != 0 || tiles / (t * passes) > 16)
+            const int s = (tiles + t * passes - 1) / (t * passes);
+            if (s > 16 || t > tiles || (!ragged && s * t * passes != tiles))
                 continue;
-            const int s = tiles / (t * passes);
             for (int xd = 1; xd >= 0; --xd) {
                 const int lds = s * t * (r + (xd ? fmx : 0)) * kTileBytes;
                 if (variant_exists(t, r, fmx, xd != 0) && lds <= kMaxLds &&
@@ -527,6 +546,7 @@ bool fit(int tiles, int fmx, int r, Plan &p)
                     p.r = r;
                     p.fmx = fmx;
                     p.xdma = xd != 0;
+                    p.ragged = s * t * passes != tiles;
                     p.lds = lds;
                     p.passes = passes;
                     return true;
@@ -539,7 +559,7 @@ bool fit(int tiles, int fmx, int r, Plan &p)
 // Rows per workgroup: the matrix split evenly over the CUs, in as few rounds as the
 // largest feasible R allows, rounded up to a multiple of 8; R is then the number of
 // 16-row groups that takes (a power of two).
-bool make_plan(int m, int n, int k, int cu_count, Plan &p)
+bool make_plan(int m, int n, int k, int cu_count, bool ragged, Plan &p)
 {
     if (k % kTileK != 0)
         return false;
@@ -547,7 +567,7 @@ bool make_plan(int m, int n, int k, int cu_count, Plan &p)
     const int fmx = m > 64 ? 4 : (m + 15) / 16;
     int rmax = 0;
     for (int r = 4; r >= 1 && rmax == 0; r >>= 1)
-        if (fit(tiles, fmx, r, p))
+        if (fit(tiles, fmx, r, ragged, p))
             rmax = r;
     if (rmax == 0)
         return false;
@@ -558,10 +578,16 @@ bool make_plan(int m, int n, int k, int cu_count, Plan &p)
     int r = 1;
     while (16 * r < rows_blk)
         r <<= 1;
-    if (!fit(tiles, fmx, r, p))  // r <= rmax, so this succeeds
+    if (!fit(tiles, fmx, r, ragged, p))  // r <= rmax, so this succeeds
         return false;
     p.rows_blk = rows_blk;
     return true;
+}
+
+// An even split of K's tiles if there is one (every slice full), else a ragged one.
+bool make_plan(int m, int n, int k, int cu_count, Plan &p)
+{
+    return make_plan(m, n, k, cu_count, false, p) || make_plan(m, n, k, cu_count, true, p);
 }
 
 template <int T, int R, int FMX, bool XDMA>
@@ -571,7 +597,7 @@ hipError_t launch_plan(const Plan &p, const void *a, const void *b, void *c, int
     if constexpr (!variant_exists(T, R, FMX, XDMA)) {
         return p.s == 0 ? hipSuccess : hipErrorInvalidConfiguration;  // never planned
     } else {
-    auto kern = skinny_kernel<T, R, FMX, XDMA>;
+    auto kern = p.ragged ? skinny_kernel<T, R, FMX, XDMA, true> : skinny_kernel<T, R, FMX, XDMA, false>;
     if (p.s == 0)  // set-up call: raise the dynamic-LDS limit of this instantiation
         return hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
     const unsigned grid = (unsigned)((n + p.rows_blk - 1) / p.rows_blk);
@@ -632,11 +658,14 @@ hipError_t skinny_init(const DeviceInfo &)
                 p.t = t;
                 p.r = r;
                 p.fmx = fmx;
-                hipError_t e = dispatch_t<true>(p, nullptr, nullptr, nullptr, 0, 0, 0, Epilogue{}, nullptr);
-                if (e == hipSuccess)
-                    e = dispatch_t<false>(p, nullptr, nullptr, nullptr, 0, 0, 0, Epilogue{}, nullptr);
-                if (e != hipSuccess)
-                    return e;
+                for (int ragged = 0; ragged < 2; ++ragged) {
+                    p.ragged = ragged != 0;
+                    hipError_t e = dispatch_t<true>(p, nullptr, nullptr, nullptr, 0, 0, 0, Epilogue{}, nullptr);
+                    if (e == hipSuccess)
+                        e = dispatch_t<false>(p, nullptr, nullptr, nullptr, 0, 0, 0, Epilogue{}, nullptr);
+                    if (e != hipSuccess)
+                        return e;
+                }
             }
     return hipSuccess;
 }

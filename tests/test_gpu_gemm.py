@@ -112,6 +112,9 @@ def test_cfg4_decode(gpu, host_threads, m, n, k):
     # workgroup per CU covers W in a single pass over K, a forced one beyond)
     (65, 4096, 4096), (128, 14336, 4096), (100, 3000, 2048), (96, 14336, 512), (128, 600, 14336),
     (200, 520, 1024), (130, 20000, 4096),
+    # K whose 128-byte tiles do not split evenly over the waves (43, 17, 74, 19, 23, 61, 5 tiles)
+    (16, 4096, 11008), (64, 4096, 11008), (1, 300, 4352), (33, 3584, 18944), (48, 1000, 4864),
+    (16, 14336, 5888), (64, 700, 15616), (100, 4096, 11008), (8, 50, 1280),
 ])
 def test_skinny_plans(gpu, host_threads, m, n, k):
     x = helpers.normal_s4(500 + m + k, m, k)
