@@ -415,6 +415,158 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
     }  // runs of rows of X
 }
 
+// ---- long-W form: many 16-row groups of W per CU and at most 16 rows of X.
+//
+// One workgroup per CU stays there and walks its groups.  Wave w owns the k range of tiles
+// [w * TW, (w + 1) * TW) of every row: its slice of X sits in registers for the whole
+// kernel, and its tiles of W pass through a ring of NBUF wave-private LDS tiles, so the
+// waves need no barrier to stream (a tile is refilled by the wave that has just consumed
+// it) and the stream never stops between groups.  A step is one tile of one group: wait
+// for it (loads complete in order: NBUF - 2 younger steps stay in flight), read its two
+// fragments, issue the load of step + NBUF - 1 into the tile consumed one step earlier,
+// multiply.  After the last tile of a group the waves leave their partial sums in one of
+// two LDS areas and meet; one wave (they take turns) adds them up and stores the 16 x 16
+// block while the others go on.  That the area of group g is free again at group g + 2
+// follows from the barrier of group g + 1, which its reducer only reaches afterwards.
+// Steps past the last group are issued like the others, as reloads of the last group
+// into tiles nobody reads, which keeps the wait counts constant.
+template <int TW, int NBUF>
+__global__ __launch_bounds__(1024) void skinny_stream_kernel(const uint8_t *__restrict__ X,
+                                                            const uint8_t *__restrict__ W,
+                                                            int32_t *__restrict__ Y, int M, int N, int K,
+                                                            int groups_per_block, Epilogue ep)
+{
+    static_assert(NBUF >= 3 && (NBUF & (NBUF - 1)) == 0, "ring positions wrap by masking");
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int waves = blockDim.x >> 6;
+    const int rowbytes = K >> 1;
+    const int groups_total = (N + 15) >> 4;
+    const int g_begin = blockIdx.x * groups_per_block;  // < groups_total by the grid's size
+    const int g_end = min(groups_total, g_begin + groups_per_block);
+    const int fr = lane & 15, fg = lane >> 4, sw = slot_swizzle(fr);
+    const int himask = (int)0xF0F0F0F0u;
+    const unsigned ring_lds = (unsigned)(size_t)I4L_LDS(lds) + wave * NBUF * kTileBytes;
+    const uint8_t *ring = lds + wave * NBUF * kTileBytes;
+    uint8_t *parts = lds + waves * NBUF * kTileBytes;  // two areas of waves * 1 KiB
+
+    v4i xg[TW][2];
+
+    // W: step (group, tile c) lands in ring position `pos`.
+    const uint8_t *wbase = W + (size_t)wave * TW * kTileRowBytes;
+    const int lrow = lane >> 3;
+    unsigned chunk[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+        chunk[u] = ((lane & 7) ^ slot_swizzle(lrow + 8 * u)) * 16;
+    auto issue = [&](int group, auto c, unsigned pos) {
+        const int g = group < g_end ? group : g_end - 1;
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int row = min(16 * g + lrow + 8 * u, N - 1);
+            // (the tile's offset goes into the scalar base, not into the instruction: the ring
+            // position is unrelated to it, and the LDS base must not go below zero)
+            dma16<true, 0>(wbase + c() * kTileRowBytes, (unsigned)row * rowbytes + chunk[u], ring_lds + pos * kTileBytes + u * 1024);
+        }
+    };
+    // The first step of W goes out ahead of X, so that the weight stream starts at once; the
+    // first wait of the loop (all but NBUF - 2 steps landed) then covers X as well.
+    static_for<NBUF - 1>([&](auto j) {
+        issue(g_begin + j() / TW, std::integral_constant<int, j() % TW>{}, (unsigned)j());
+        if constexpr (j() == 0) {
+            // X: fragment form, once.
+            const uint8_t *xbase = X + (size_t)wave * TW * kTileRowBytes;
+            const unsigned x_off = (unsigned)(fr < M ? fr : M - 1) * rowbytes + fg * 16;
+            static_for<2 * TW>([&](auto q) {
+                load16_untracked<(q() >> 1) * kTileRowBytes + (q() & 1) * 64>(xg[q() >> 1][q() & 1], xbase, x_off);
+            });
+        }
+    });
+
+    v4i acc = {0, 0, 0, 0};
+    unsigned pos = 0;  // ring position of the current step
+    int reducer = 0;   // wave that adds up the current group
+#pragma unroll 1
+    for (int g = g_begin; g < g_end; ++g) {
+        // (the shift count and mask are hidden from the optimiser in every group: widened
+        // once outside the loop, X would take three times the registers)
+        int shift = 4, mask = himask;
+        asm volatile("" : "+s"(shift), "+s"(mask));
+        static_for<TW>([&](auto c) {
+            wait_vm_imm<2 * (NBUF - 2)>();
+            if constexpr (c() == 0) {
+                // (needed once, after the first wait; it costs nothing to say it per group)
+#pragma unroll
+                for (int cc = 0; cc < TW; ++cc)
+#pragma unroll
+                    for (int s = 0; s < 2; ++s)
+                        settle(xg[cc][s]);
+            }
+            v4i w[2];
+#pragma unroll
+            for (int s = 0; s < 2; ++s)
+                w[s] = *(const v4i *)(ring + pos * kTileBytes + fr * kTileRowBytes + (((4 * s + fg) ^ sw) * 16));
+            constexpr int ahead = c() + NBUF - 1;
+            issue(g + ahead / TW, std::integral_constant<int, ahead % TW>{}, (pos + NBUF - 1) & (NBUF - 1));
+            pos = (pos + 1) & (NBUF - 1);
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                const v4i x = xg[c()][s];
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8((w[s] << 4) & himask, (x << shift) & mask, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[s] & himask, x & mask, acc, 0, 0, 0);
+            }
+        });
+        // Partial sums, in the layout that lets the reducing lane 4 * m + j fetch
+        // (fr = m, fg = j) without bank conflicts.
+        v4i *area = (v4i *)(parts + (g & 1) * waves * 1024);
+        area[wave * 64 + 16 * fg + (fr ^ (2 * fg))] = acc;
+        acc = (v4i){0, 0, 0, 0};
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if (wave == reducer) {
+            const int om = lane >> 2, oj = lane & 3;
+            const v4i *p = area + 16 * oj + (om ^ (2 * oj));
+            // four reads in flight at a time (this wave is off the others' critical path, and
+            // its registers hold the X fragments)
+            v4i sum = {0, 0, 0, 0};
+#pragma unroll 1
+            for (int w0 = 0; w0 < waves; w0 += 4) {
+                v4i part[4];
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    part[q] = p[(w0 + q < waves ? w0 + q : 0) * 64];
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    sum += w0 + q < waves ? part[q] : (v4i){0, 0, 0, 0};
+            }
+            sum = sum >> 8;  // both operands carried a factor 16
+            const int m = om, n = 16 * g + 4 * oj;
+            if (m < M) {
+                const float rs = ep.row_scale ? ep.row_scale[m] : 1.f;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int nn = n + q < N ? n + q : N - 1;
+                    sum[q] = epilogue_value(ep, sum[q], ep.bias ? ep.bias[nn] : 0, rs,
+                                            ep.col_scale ? ep.col_scale[nn] : 1.f);
+                }
+                int32_t *dst = Y + (size_t)m * N + n;
+                if (n + 3 < N && (N & 3) == 0) {
+                    *(v4i *)dst = sum;
+                } else {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                        if (n + q < N)
+                            dst[q] = sum[q];
+                }
+            }
+        }
+        reducer = reducer + 1 == waves ? 0 : reducer + 1;
+    }
+    wait_vm_imm<0>();  // the reloads past the last group land before the LDS is given up
+}
+
 // ---- fallback for K that is a multiple of 128 but does not split into tiles: the
 //      straightforward version (fragment-layout global loads, 128 nibbles per step).
 template <int FMX, int WAVES>
@@ -646,8 +798,85 @@ hipError_t dispatch_t(const Plan &p, const void *a, const void *b, void *c, int 
 
 }  // namespace
 
+namespace {
+
+// The long-W form: at most 16 rows of X, K in whole tiles that split evenly over at most 16
+// waves with at most 8 tiles each, W below 4 GiB (32-bit lane offsets), and enough 16-row
+// groups per CU that a workgroup which stays on its CU beats one workgroup per 64 rows.
+constexpr int kStreamMinGroupsPerCu = 5;  // measured crossover: the other form wins while one workgroup of 64 rows per CU covers W
+
+struct StreamPlan {
+    int tw = 0, s = 0, bufs = 4, groups_per_block = 0, grid = 0, lds = 0;
+};
+
+bool make_stream_plan(int m, int n, int k, int cu_count, StreamPlan &p)
+{
+    if (m > 16 || k % kTileK != 0 || cu_count <= 0 || (unsigned long long)n * (unsigned long long)(k >> 1) >= (1ull << 32))
+        return false;
+    const int tiles = k / kTileK;
+    // Most waves first, but at least two tiles per wave if possible: with one, the waves
+    // meet after every step.
+    int s = 0;
+    for (int min_tw = 2; min_tw >= 1 && s == 0; --min_tw)
+        for (int cand = 16; cand >= 1 && s == 0; --cand)
+            if (tiles % cand == 0 && tiles / cand <= 8 && tiles / cand >= min_tw)
+                s = cand;
+    if (s == 0)
+        return false;
+    const int groups = (n + 15) / 16;
+    if (groups < kStreamMinGroupsPerCu * cu_count)
+        return false;
+    p.tw = tiles / s;
+    p.s = s;
+    p.groups_per_block = (groups + cu_count - 1) / cu_count;
+    p.grid = (groups + p.groups_per_block - 1) / p.groups_per_block;
+    p.bufs = s <= 8 ? 8 : 4;  // up to eight waves: a deeper ring keeps as many bytes in flight
+    p.lds = s * p.bufs * kTileBytes + 2 * s * 1024;
+    return p.lds <= kMaxLds;
+}
+
+template <int TW>
+hipError_t launch_stream(const StreamPlan &p, const void *a, const void *b, void *c, int m, int n, int k,
+                         const Epilogue &ep, hipStream_t stream)
+{
+    auto kern = p.bufs == 8 ? skinny_stream_kernel<TW, 8> : skinny_stream_kernel<TW, 4>;
+    if (p.s == 0)  // set-up call
+        return hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
+    kern<<<p.grid, p.s * 64, p.lds, stream>>>((const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k,
+                                               p.groups_per_block, ep);
+    return hipGetLastError();
+}
+
+hipError_t dispatch_stream(const StreamPlan &p, const void *a, const void *b, void *c, int m, int n, int k,
+                           const Epilogue &ep, hipStream_t stream)
+{
+    switch (p.tw) {
+    case 1: return launch_stream<1>(p, a, b, c, m, n, k, ep, stream);
+    case 2: return launch_stream<2>(p, a, b, c, m, n, k, ep, stream);
+    case 3: return launch_stream<3>(p, a, b, c, m, n, k, ep, stream);
+    case 4: return launch_stream<4>(p, a, b, c, m, n, k, ep, stream);
+    case 5: return launch_stream<5>(p, a, b, c, m, n, k, ep, stream);
+    case 6: return launch_stream<6>(p, a, b, c, m, n, k, ep, stream);
+    case 7: return launch_stream<7>(p, a, b, c, m, n, k, ep, stream);
+    case 8: return launch_stream<8>(p, a, b, c, m, n, k, ep, stream);
+    default: return hipErrorInvalidConfiguration;
+    }
+}
+
+}  // namespace
+
 hipError_t skinny_init(const DeviceInfo &)
 {
+    for (int tw = 1; tw <= 8; ++tw) {
+        for (int bufs = 4; bufs <= 8; bufs += 4) {
+            StreamPlan sp;  // s == 0: set-up call
+            sp.tw = tw;
+            sp.bufs = bufs;
+            const hipError_t e = dispatch_stream(sp, nullptr, nullptr, nullptr, 0, 0, 0, Epilogue{}, nullptr);
+            if (e != hipSuccess)
+                return e;
+        }
+    }
     // Every instantiation may use up to the full LDS of a CU (a plan with s == 0 is the
     // set-up call of launch_plan).
     for (int t = 1; t <= 4; ++t)
@@ -701,6 +930,9 @@ bool skinny_preferred(int m, int n, int k, const DeviceInfo &dev)
 hipError_t launch_skinny(const void *a, const void *b, void *c, int m, int n, int k,
                          const Epilogue &ep, const DeviceInfo &dev, hipStream_t stream)
 {
+    StreamPlan sp;
+    if (make_stream_plan(m, n, k, dev.cu_count, sp))
+        return dispatch_stream(sp, a, b, c, m, n, k, ep, stream);
     Plan p;
     if (make_plan(m, n, k, dev.cu_count, p))
         return p.xdma ? dispatch_t<true>(p, a, b, c, m, n, k, ep, stream)
