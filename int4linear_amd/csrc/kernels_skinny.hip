@@ -800,8 +800,8 @@ hipError_t dispatch_t(const Plan &p, const void *a, const void *b, void *c, int 
 
 namespace {
 
-// The long-W form: at most 16 rows of X, K in whole tiles that split evenly over at most 16
-// waves with at most 8 tiles each, W below 4 GiB (32-bit lane offsets), and enough 16-row
+// The long-W form: at most 16 rows of X, K in whole tiles that split evenly over 7 to 16
+// waves with 2 to 8 tiles each, W below 4 GiB (32-bit lane offsets), and enough 16-row
 // groups per CU that a workgroup which stays on its CU beats one workgroup per 64 rows.
 constexpr int kStreamMinGroupsPerCu = 5;  // measured crossover: the other form wins while one workgroup of 64 rows per CU covers W
 
@@ -816,11 +816,13 @@ bool make_stream_plan(int m, int n, int k, int cu_count, StreamPlan &p)
     const int tiles = k / kTileK;
     // Most waves first, but at least two tiles per wave if possible: with one, the waves
     // meet after every step.
+    // Most waves first.  At least seven of them, with at least two tiles each: with fewer waves
+    // the stream does not keep going, and with one tile the waves meet after every step
+    // (measured: K up to 3072 is faster in the other form).
     int s = 0;
-    for (int min_tw = 2; min_tw >= 1 && s == 0; --min_tw)
-        for (int cand = 16; cand >= 1 && s == 0; --cand)
-            if (tiles % cand == 0 && tiles / cand <= 8 && tiles / cand >= min_tw)
-                s = cand;
+    for (int cand = 16; cand >= 7 && s == 0; --cand)
+        if (tiles % cand == 0 && tiles / cand <= 8 && tiles / cand >= 2)
+            s = cand;
     if (s == 0)
         return false;
     const int groups = (n + 15) / 16;
@@ -851,7 +853,6 @@ hipError_t dispatch_stream(const StreamPlan &p, const void *a, const void *b, vo
                            const Epilogue &ep, hipStream_t stream)
 {
     switch (p.tw) {
-    case 1: return launch_stream<1>(p, a, b, c, m, n, k, ep, stream);
     case 2: return launch_stream<2>(p, a, b, c, m, n, k, ep, stream);
     case 3: return launch_stream<3>(p, a, b, c, m, n, k, ep, stream);
     case 4: return launch_stream<4>(p, a, b, c, m, n, k, ep, stream);
@@ -867,7 +868,7 @@ hipError_t dispatch_stream(const StreamPlan &p, const void *a, const void *b, vo
 
 hipError_t skinny_init(const DeviceInfo &)
 {
-    for (int tw = 1; tw <= 8; ++tw) {
+    for (int tw = 2; tw <= 8; ++tw) {
         for (int bufs = 4; bufs <= 8; bufs += 4) {
             StreamPlan sp;  // s == 0: set-up call
             sp.tw = tw;

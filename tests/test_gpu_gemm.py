@@ -116,9 +116,11 @@ def test_cfg4_decode(gpu, host_threads, m, n, k):
     (16, 4096, 11008), (64, 4096, 11008), (1, 300, 4352), (33, 3584, 18944), (48, 1000, 4864),
     (16, 14336, 5888), (64, 700, 15616), (100, 4096, 11008), (8, 50, 1280),
     # at most 16 rows of X against more than 64 rows of W per CU: the form whose workgroups stay on
-    # their CU and stream W through wave-private rings (1, 2, 4, 7 and 5 tiles per wave)
-    (16, 20500, 256), (1, 21000, 512), (7, 20481, 1024), (16, 20480, 4096), (5, 21001, 1792),
-    (16, 20480, 14336), (16, 33000, 5120), (3, 40001, 2048),
+    # their CU and stream W through wave-private rings (2 to 8 tiles for each of 7 to 16 waves)
+    (16, 20480, 4096), (5, 21001, 3584), (16, 20480, 14336), (16, 33000, 5120), (3, 40001, 7168),
+    (1, 21000, 6144), (9, 20481, 8192), (16, 20500, 28672), (2, 20490, 32768),
+    # ... and shapes with as many rows of W whose K does not qualify
+    (16, 20500, 256), (7, 20481, 1024), (3, 40001, 2048),
 ])
 def test_skinny_plans(gpu, host_threads, m, n, k):
     x = helpers.normal_s4(500 + m + k, m, k)
@@ -179,7 +181,7 @@ def test_ragged_k_runs_on_the_fp6_kernel(gpu, host_threads, m, n, k):
     (16, 1024, 1024, ("auto", "skinny", "mfma", "fp6")),
     (40, 515, 14336, ("skinny",)),
     (100, 4100, 4096, ("auto", "skinny")),   # two runs of rows of X: the row scales move with them
-    (13, 20600, 1024, ("auto", "skinny")),   # the form for very many rows of W
+    (13, 20600, 4096, ("auto", "skinny")),   # the form for very many rows of W
     (33, 70, 72, ("auto", "simple", "fp6")),
     (9, 1000, 1920, ("skinny",)),           # the fallback streaming kernel
     (2048, 2304, 1024, ("auto", "mfma")),   # 72 tiles of 256 x 256, several per workgroup
