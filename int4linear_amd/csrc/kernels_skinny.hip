@@ -1,4 +1,8 @@
-// Weight-streaming kernels for skinny M (M <= 64): the decode-shaped linear layer.
+// Weight-streaming kernels for skinny M: the decode-shaped linear layer.  Three kernels:
+// skinny_kernel (up to 64 rows of X per run, W's rows split over one workgroup per CU and
+// per 64 rows), skinny_stream_kernel (at most 16 rows of X against very many rows of W:
+// workgroups that stay on their CU) and skinny_basic_kernel (K that is not a whole number
+// of 128-byte tiles).
 //
 // The job is HBM-bound: every byte of W (N x K/2) is read exactly once and the arithmetic
 // (v_mfma_i32_16x16x64_i8 after the same 16x nibble widening as the big int8 kernel:
