@@ -1,7 +1,7 @@
 // Weight-streaming kernels for skinny M: the decode-shaped linear layer.  Three kernels:
 // skinny_kernel (up to 64 rows of X per run, W's rows split over one workgroup per CU and
-// per 64 rows), skinny_stream_kernel (at most 16 rows of X against very many rows of W:
-// workgroups that stay on their CU) and skinny_basic_kernel (K that is not a whole number
+// per 64 rows), skinny_stream_kernel (very many rows of W: workgroups that stay on their
+// CU) and skinny_basic_kernel (K that is not a whole number
 // of 128-byte tiles).
 //
 // The job is HBM-bound: every byte of W (N x K/2) is read exactly once and the arithmetic
@@ -419,7 +419,7 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
     }  // runs of rows of X
 }
 
-// ---- long-W form: many 16-row groups of W per CU and at most 16 rows of X.
+// ---- long-W form: many 16-row groups of W per CU, FMX 16-row groups of X.
 //
 // One workgroup per CU stays there and walks its groups.  Wave w owns the k range of tiles
 // [w * TW, (w + 1) * TW) of every row: its slice of X sits in registers for the whole
@@ -434,8 +434,8 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
 // follows from the barrier of group g + 1, which its reducer only reaches afterwards.
 // Steps past the last group are issued like the others, as reloads of the last group
 // into tiles nobody reads, which keeps the wait counts constant.
-template <int TW, int NBUF>
-__global__ __launch_bounds__(1024) void skinny_stream_kernel(const uint8_t *__restrict__ X,
+template <int TW, int NBUF, int FMX>
+__global__ __launch_bounds__(FMX == 1 ? 1024 : 512) void skinny_stream_kernel(const uint8_t *__restrict__ X,
                                                             const uint8_t *__restrict__ W,
                                                             int32_t *__restrict__ Y, int M, int N, int K,
                                                             int groups_per_block, Epilogue ep)
@@ -453,9 +453,18 @@ __global__ __launch_bounds__(1024) void skinny_stream_kernel(const uint8_t *__re
     const int himask = (int)0xF0F0F0F0u;
     const unsigned ring_lds = (unsigned)(size_t)I4L_LDS(lds) + wave * NBUF * kTileBytes;
     const uint8_t *ring = lds + wave * NBUF * kTileBytes;
-    uint8_t *parts = lds + waves * NBUF * kTileBytes;  // two areas of waves * 1 KiB
+    // Partial sums: FMX KiB per wave.  With one row group of X there are two such areas, used
+    // by alternate groups of W (one meeting per group); with more there is one (and a second
+    // meeting per group, after the partial sums have been read).
+    constexpr bool kTwoAreas = FMX == 1;
+    uint8_t *parts = lds + waves * NBUF * kTileBytes;
 
-    v4i xg[TW][2];
+    // X fragments: packed as loaded and widened at every use, or, where the 256 registers of
+    // the eight-wave form have room for it, widened once (several row groups of X make the
+    // widening the bottleneck otherwise).
+    constexpr bool kKeepWide = FMX > 1 && TW * FMX <= 8;
+    v4i xg[TW][2][FMX];
+    v4i xw[kKeepWide ? TW : 1][2][kKeepWide ? FMX : 1][2];
 
     // W: step (group, tile c) lands in ring position `pos`.
     const uint8_t *wbase = W + (size_t)wave * TW * kTileRowBytes;
@@ -481,16 +490,23 @@ __global__ __launch_bounds__(1024) void skinny_stream_kernel(const uint8_t *__re
         if constexpr (j() == 0) {
             // X: fragment form, once.
             const uint8_t *xbase = X + (size_t)wave * TW * kTileRowBytes;
-            const unsigned x_off = (unsigned)(fr < M ? fr : M - 1) * rowbytes + fg * 16;
-            static_for<2 * TW>([&](auto q) {
-                load16_untracked<(q() >> 1) * kTileRowBytes + (q() & 1) * 64>(xg[q() >> 1][q() & 1], xbase, x_off);
-            });
+#pragma unroll
+            for (int f = 0; f < FMX; ++f) {
+                const int xr = 16 * f + fr;
+                const unsigned x_off = (unsigned)(xr < M ? xr : M - 1) * rowbytes + fg * 16;
+                static_for<2 * TW>([&](auto q) {
+                    load16_untracked<(q() >> 1) * kTileRowBytes + (q() & 1) * 64>(xg[q() >> 1][q() & 1][f], xbase, x_off);
+                });
+            }
         }
     });
 
-    v4i acc = {0, 0, 0, 0};
+    v4i acc[FMX];
+#pragma unroll
+    for (int f = 0; f < FMX; ++f)
+        acc[f] = (v4i){0, 0, 0, 0};
     unsigned pos = 0;  // ring position of the current step
-    int reducer = 0;   // wave that adds up the current group
+    int reducer = 0;   // first of the FMX waves that add up the current group
 #pragma unroll 1
     for (int g = g_begin; g < g_end; ++g) {
         // (the shift count and mask are hidden from the optimiser in every group: widened
@@ -505,7 +521,22 @@ __global__ __launch_bounds__(1024) void skinny_stream_kernel(const uint8_t *__re
                 for (int cc = 0; cc < TW; ++cc)
 #pragma unroll
                     for (int s = 0; s < 2; ++s)
-                        settle(xg[cc][s]);
+#pragma unroll
+                        for (int f = 0; f < FMX; ++f)
+                            settle(xg[cc][s][f]);
+                if constexpr (kKeepWide) {
+                    if (g == g_begin) {
+#pragma unroll
+                        for (int cc = 0; cc < TW; ++cc)
+#pragma unroll
+                            for (int s = 0; s < 2; ++s)
+#pragma unroll
+                                for (int f = 0; f < FMX; ++f) {
+                                    xw[cc][s][f][0] = (xg[cc][s][f] << 4) & himask;
+                                    xw[cc][s][f][1] = xg[cc][s][f] & himask;
+                                }
+                    }
+                }
             }
             v4i w[2];
 #pragma unroll
@@ -516,22 +547,38 @@ __global__ __launch_bounds__(1024) void skinny_stream_kernel(const uint8_t *__re
             pos = (pos + 1) & (NBUF - 1);
 #pragma unroll
             for (int s = 0; s < 2; ++s) {
-                const v4i x = xg[c()][s];
-                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8((w[s] << 4) & himask, (x << shift) & mask, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[s] & himask, x & mask, acc, 0, 0, 0);
+                const v4i wlo = (w[s] << 4) & himask, whi = w[s] & himask;
+#pragma unroll
+                for (int f = 0; f < FMX; ++f) {
+                    if constexpr (kKeepWide) {
+                        acc[f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo, xw[c()][s][f][0], acc[f], 0, 0, 0);
+                        acc[f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi, xw[c()][s][f][1], acc[f], 0, 0, 0);
+                    } else {
+                        const v4i x = xg[c()][s][f];
+                        acc[f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo, (x << shift) & mask, acc[f], 0, 0, 0);
+                        acc[f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi, x & mask, acc[f], 0, 0, 0);
+                    }
+                }
             }
         });
         // Partial sums, in the layout that lets the reducing lane 4 * m + j fetch
         // (fr = m, fg = j) without bank conflicts.
-        v4i *area = (v4i *)(parts + (g & 1) * waves * 1024);
-        area[wave * 64 + 16 * fg + (fr ^ (2 * fg))] = acc;
-        acc = (v4i){0, 0, 0, 0};
+        v4i *area = (v4i *)(parts + (kTwoAreas ? (g & 1) * waves * 1024 : 0));
+#pragma unroll
+        for (int f = 0; f < FMX; ++f) {
+            area[(wave * FMX + f) * 64 + 16 * fg + (fr ^ (2 * fg))] = acc[f];
+            acc[f] = (v4i){0, 0, 0, 0};
+        }
         __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        if (wave == reducer) {
+        // Waves reducer, reducer + 1, ... (mod S) take one 16 x 16 block each.
+        int f_mine = wave - reducer;
+        if (f_mine < 0)
+            f_mine += waves;
+        if (f_mine < FMX) {
             const int om = lane >> 2, oj = lane & 3;
-            const v4i *p = area + 16 * oj + (om ^ (2 * oj));
+            const v4i *p = area + f_mine * 64 + 16 * oj + (om ^ (2 * oj));
             // four reads in flight at a time (this wave is off the others' critical path, and
             // its registers hold the X fragments)
             v4i sum = {0, 0, 0, 0};
@@ -540,13 +587,13 @@ __global__ __launch_bounds__(1024) void skinny_stream_kernel(const uint8_t *__re
                 v4i part[4];
 #pragma unroll
                 for (int q = 0; q < 4; ++q)
-                    part[q] = p[(w0 + q < waves ? w0 + q : 0) * 64];
+                    part[q] = p[(w0 + q < waves ? w0 + q : 0) * FMX * 64];
 #pragma unroll
                 for (int q = 0; q < 4; ++q)
                     sum += w0 + q < waves ? part[q] : (v4i){0, 0, 0, 0};
             }
             sum = sum >> 8;  // both operands carried a factor 16
-            const int m = om, n = 16 * g + 4 * oj;
+            const int m = 16 * f_mine + om, n = 16 * g + 4 * oj;
             if (m < M) {
                 const float rs = ep.row_scale ? ep.row_scale[m] : 1.f;
 #pragma unroll
@@ -566,7 +613,13 @@ __global__ __launch_bounds__(1024) void skinny_stream_kernel(const uint8_t *__re
                 }
             }
         }
-        reducer = reducer + 1 == waves ? 0 : reducer + 1;
+        if (!kTwoAreas) {
+            // the partial sums have been read: the area may be written again
+            __builtin_amdgcn_s_waitcnt(0xC07F);
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+        }
+        reducer = reducer + FMX >= waves ? reducer + FMX - waves : reducer + FMX;
     }
     wait_vm_imm<0>();  // the reloads past the last group land before the LDS is given up
 }
@@ -804,66 +857,85 @@ hipError_t dispatch_t(const Plan &p, const void *a, const void *b, void *c, int 
 
 namespace {
 
-// The long-W form: at most 16 rows of X, K in whole tiles that split evenly over 7 to 16
-// waves with 2 to 8 tiles each, W below 4 GiB (32-bit lane offsets), and enough 16-row
-// groups per CU that a workgroup which stays on its CU beats one workgroup per 64 rows.
-constexpr int kStreamMinGroupsPerCu = 5;  // measured crossover: the other form wins while one workgroup of 64 rows per CU covers W
+// The long-W form: K in whole tiles that split evenly over the waves with 2 to 8 tiles each
+// (with one tile the waves meet after every step), W below 4 GiB (32-bit lane offsets), and
+// enough 16-row groups per CU that a workgroup which stays on its CU beats one workgroup
+// per 64 rows.  At most 16 rows of X: 7 to 16 waves, most waves first (with fewer the stream
+// does not keep going: K up to 3072 is faster in the other form).  17 to 64 rows: 7 or 8
+// waves (256 registers each for the X fragments, TW * FMX <= 16 of them per step parity)
+// and an eight-tile ring.
+constexpr int kStreamMinGroupsPerCu = 5;       // measured crossover at up to 16 rows of X
+constexpr int kStreamMinGroupsPerCuWide = 8;   // ... with more rows (X is loaded once per workgroup, in fragment form)
 
 struct StreamPlan {
-    int tw = 0, s = 0, bufs = 4, groups_per_block = 0, grid = 0, lds = 0;
+    int tw = 0, s = 0, fmx = 1, bufs = 4, groups_per_block = 0, grid = 0, lds = 0;
 };
 
 bool make_stream_plan(int m, int n, int k, int cu_count, StreamPlan &p)
 {
-    if (m > 16 || k % kTileK != 0 || cu_count <= 0 || (unsigned long long)n * (unsigned long long)(k >> 1) >= (1ull << 32))
+    if (m > 64 || k % kTileK != 0 || cu_count <= 0 || (unsigned long long)n * (unsigned long long)(k >> 1) >= (1ull << 32))
         return false;
     const int tiles = k / kTileK;
-    // Most waves first, but at least two tiles per wave if possible: with one, the waves
-    // meet after every step.
-    // Most waves first.  At least seven of them, with at least two tiles each: with fewer waves
-    // the stream does not keep going, and with one tile the waves meet after every step
-    // (measured: K up to 3072 is faster in the other form).
+    const int fmx = (m + 15) / 16;
     int s = 0;
-    for (int cand = 16; cand >= 7 && s == 0; --cand)
-        if (tiles % cand == 0 && tiles / cand <= 8 && tiles / cand >= 2)
+    for (int cand = fmx == 1 ? 16 : 8; cand >= 7 && s == 0; --cand)
+        if (tiles % cand == 0 && tiles / cand <= 8 && tiles / cand >= 2 && (fmx == 1 || tiles / cand * fmx <= 16))
             s = cand;
     if (s == 0)
         return false;
     const int groups = (n + 15) / 16;
-    if (groups < kStreamMinGroupsPerCu * cu_count)
+    if (groups < (fmx == 1 ? kStreamMinGroupsPerCu : kStreamMinGroupsPerCuWide) * cu_count)
         return false;
     p.tw = tiles / s;
     p.s = s;
+    p.fmx = fmx;
     p.groups_per_block = (groups + cu_count - 1) / cu_count;
     p.grid = (groups + p.groups_per_block - 1) / p.groups_per_block;
     p.bufs = s <= 8 ? 8 : 4;  // up to eight waves: a deeper ring keeps as many bytes in flight
-    p.lds = s * p.bufs * kTileBytes + 2 * s * 1024;
+    p.lds = s * p.bufs * kTileBytes + (fmx == 1 ? 2 : fmx) * s * 1024;
     return p.lds <= kMaxLds;
 }
 
-template <int TW>
+template <int TW, int FMX>
 hipError_t launch_stream(const StreamPlan &p, const void *a, const void *b, void *c, int m, int n, int k,
                          const Epilogue &ep, hipStream_t stream)
 {
-    auto kern = p.bufs == 8 ? skinny_stream_kernel<TW, 8> : skinny_stream_kernel<TW, 4>;
-    if (p.s == 0)  // set-up call
-        return hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
-    kern<<<p.grid, p.s * 64, p.lds, stream>>>((const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k,
-                                               p.groups_per_block, ep);
-    return hipGetLastError();
+    if constexpr (FMX > 1 && TW * FMX > 16) {
+        return p.s == 0 ? hipSuccess : hipErrorInvalidConfiguration;  // never planned
+    } else {
+        auto kern = (FMX == 1 && p.bufs == 4) ? skinny_stream_kernel<TW, 4, FMX> : skinny_stream_kernel<TW, 8, FMX>;
+        if (p.s == 0)  // set-up call
+            return hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
+        kern<<<p.grid, p.s * 64, p.lds, stream>>>((const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k,
+                                                   p.groups_per_block, ep);
+        return hipGetLastError();
+    }
+}
+
+template <int TW>
+hipError_t dispatch_stream_f(const StreamPlan &p, const void *a, const void *b, void *c, int m, int n, int k,
+                             const Epilogue &ep, hipStream_t stream)
+{
+    switch (p.fmx) {
+    case 1: return launch_stream<TW, 1>(p, a, b, c, m, n, k, ep, stream);
+    case 2: return launch_stream<TW, 2>(p, a, b, c, m, n, k, ep, stream);
+    case 3: return launch_stream<TW, 3>(p, a, b, c, m, n, k, ep, stream);
+    case 4: return launch_stream<TW, 4>(p, a, b, c, m, n, k, ep, stream);
+    default: return hipErrorInvalidConfiguration;
+    }
 }
 
 hipError_t dispatch_stream(const StreamPlan &p, const void *a, const void *b, void *c, int m, int n, int k,
                            const Epilogue &ep, hipStream_t stream)
 {
     switch (p.tw) {
-    case 2: return launch_stream<2>(p, a, b, c, m, n, k, ep, stream);
-    case 3: return launch_stream<3>(p, a, b, c, m, n, k, ep, stream);
-    case 4: return launch_stream<4>(p, a, b, c, m, n, k, ep, stream);
-    case 5: return launch_stream<5>(p, a, b, c, m, n, k, ep, stream);
-    case 6: return launch_stream<6>(p, a, b, c, m, n, k, ep, stream);
-    case 7: return launch_stream<7>(p, a, b, c, m, n, k, ep, stream);
-    case 8: return launch_stream<8>(p, a, b, c, m, n, k, ep, stream);
+    case 2: return dispatch_stream_f<2>(p, a, b, c, m, n, k, ep, stream);
+    case 3: return dispatch_stream_f<3>(p, a, b, c, m, n, k, ep, stream);
+    case 4: return dispatch_stream_f<4>(p, a, b, c, m, n, k, ep, stream);
+    case 5: return dispatch_stream_f<5>(p, a, b, c, m, n, k, ep, stream);
+    case 6: return dispatch_stream_f<6>(p, a, b, c, m, n, k, ep, stream);
+    case 7: return dispatch_stream_f<7>(p, a, b, c, m, n, k, ep, stream);
+    case 8: return dispatch_stream_f<8>(p, a, b, c, m, n, k, ep, stream);
     default: return hipErrorInvalidConfiguration;
     }
 }
@@ -873,14 +945,16 @@ hipError_t dispatch_stream(const StreamPlan &p, const void *a, const void *b, vo
 hipError_t skinny_init(const DeviceInfo &)
 {
     for (int tw = 2; tw <= 8; ++tw) {
-        for (int bufs = 4; bufs <= 8; bufs += 4) {
-            StreamPlan sp;  // s == 0: set-up call
-            sp.tw = tw;
-            sp.bufs = bufs;
-            const hipError_t e = dispatch_stream(sp, nullptr, nullptr, nullptr, 0, 0, 0, Epilogue{}, nullptr);
-            if (e != hipSuccess)
-                return e;
-        }
+        for (int fmx = 1; fmx <= 4; ++fmx)
+            for (int bufs = 4; bufs <= 8; bufs += 4) {
+                StreamPlan sp;  // s == 0: set-up call
+                sp.tw = tw;
+                sp.fmx = fmx;
+                sp.bufs = bufs;
+                const hipError_t e = dispatch_stream(sp, nullptr, nullptr, nullptr, 0, 0, 0, Epilogue{}, nullptr);
+                if (e != hipSuccess)
+                    return e;
+            }
     }
     // Every instantiation may use up to the full LDS of a CU (a plan with s == 0 is the
     // set-up call of launch_plan).

@@ -119,8 +119,10 @@ def test_cfg4_decode(gpu, host_threads, m, n, k):
     # their CU and stream W through wave-private rings (2 to 8 tiles for each of 7 to 16 waves)
     (16, 20480, 4096), (5, 21001, 3584), (16, 20480, 14336), (16, 33000, 5120), (3, 40001, 7168),
     (1, 21000, 6144), (9, 20481, 8192), (16, 20500, 28672), (2, 20490, 32768),
+    # ... the same with 17 to 64 rows of X (seven or eight waves, widened X kept where it fits)
+    (64, 32800, 4096), (33, 32768, 8192), (48, 33000, 3584), (17, 32770, 7168), (32, 32768, 14336),
     # ... and shapes with as many rows of W whose K does not qualify
-    (16, 20500, 256), (7, 20481, 1024), (3, 40001, 2048),
+    (16, 20500, 256), (7, 20481, 1024), (3, 40001, 2048), (64, 32768, 14336), (40, 33000, 5120),
 ])
 def test_skinny_plans(gpu, host_threads, m, n, k):
     x = helpers.normal_s4(500 + m + k, m, k)
@@ -182,6 +184,7 @@ def test_ragged_k_runs_on_the_fp6_kernel(gpu, host_threads, m, n, k):
     (40, 515, 14336, ("skinny",)),
     (100, 4100, 4096, ("auto", "skinny")),   # two runs of rows of X: the row scales move with them
     (13, 20600, 4096, ("auto", "skinny")),   # the form for very many rows of W
+    (50, 32790, 4096, ("auto", "skinny")),   # ... with several row groups of X
     (33, 70, 72, ("auto", "simple", "fp6")),
     (9, 1000, 1920, ("skinny",)),           # the fallback streaming kernel
     (2048, 2304, 1024, ("auto", "mfma")),   # 72 tiles of 256 x 256, several per workgroup
