@@ -865,7 +865,7 @@ namespace {
 // waves (256 registers each for the X fragments, TW * FMX <= 16 of them per step parity)
 // and an eight-tile ring.
 constexpr int kStreamMinGroupsPerCu = 5;       // measured crossover at up to 16 rows of X
-constexpr int kStreamMinGroupsPerCuWide = 8;   // ... with more rows (X is loaded once per workgroup, in fragment form)
+constexpr int kStreamMinGroupsPerCuWide = 8;   // ... with more rows of X and more than two tiles per wave
 
 struct StreamPlan {
     int tw = 0, s = 0, fmx = 1, bufs = 4, groups_per_block = 0, grid = 0, lds = 0;
@@ -884,7 +884,7 @@ bool make_stream_plan(int m, int n, int k, int cu_count, StreamPlan &p)
     if (s == 0)
         return false;
     const int groups = (n + 15) / 16;
-    if (groups < (fmx == 1 ? kStreamMinGroupsPerCu : kStreamMinGroupsPerCuWide) * cu_count)
+    if (groups < (fmx == 1 || tiles / s <= 2 ? kStreamMinGroupsPerCu : kStreamMinGroupsPerCuWide) * cu_count)
         return false;
     p.tw = tiles / s;
     p.s = s;
