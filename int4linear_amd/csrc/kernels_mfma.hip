@@ -387,6 +387,9 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
     constexpr int kDmaStride = kPositions / C::CH;   // CH/2 loads x 2 wave parities per half
     static_assert(C::CH % 2 == 0 && kDmaStride >= 1 && kDmaStride * C::CH == kPositions,
                   "load spreading needs CH places per half");
+    // X fragment 0 of the next unit is read with part 1 and widened during this unit's last
+    // step, so part 1 must go out before that step begins.
+    static_assert(kPositions / kReadParts + 1 < (C::FM - 1) * kSlots, "part 1 of the LDS reads comes too late");
     const int wave_par = wave & 1;
     // Housekeeping common to both halves at position (j, slot): `read_ring`/`read_h` name the
     // unit whose fragments are read, `half_pos` is 0 in the second half of an iteration,
