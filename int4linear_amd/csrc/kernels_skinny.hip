@@ -197,6 +197,9 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
     constexpr bool kPairX = !XDMA && T % 2 == 0;
     // Row groups of W issued before X: the weight stream starts at once, X follows.
     constexpr int kGroupsBeforeX = (!XDMA && R > 1) ? 1 : 0;
+    // With a single row group its first tile goes out before X for the same reason (the
+    // waits below need no change: X then sits right behind that tile).
+    constexpr int kTilesBeforeX = (!XDMA && R == 1 && T > 1) ? 1 : 0;
     v4i xg[XDMA ? 1 : T][2][FMX];
     v4i acc[R][FMX];
 #pragma unroll
@@ -250,16 +253,23 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
         const size_t kbyte0 = (size_t)(first_tile - skip) * kTileRowBytes;
         const uint8_t *wbase = W + (size_t)n0 * rowbytes + kbyte0;
         const uint8_t *xbase = X + kbyte0;
-        auto issue_w = [&](int rg) {
-            static_for<T>([&](auto t) {
+        auto issue_w = [&](int rg, auto first, auto count) {  // tiles first .. first + count - 1 of group rg
+            static_for<count()>([&](auto i) {
+                constexpr int t = first() + i();
 #pragma unroll
                 for (int u = 0; u < 2; ++u)
-                    dma16<true, t() * kTileRowBytes>(wbase, w_off[rg][u], my_lds + (rg * T + t()) * kTileBytes + u * 1024);
+                    dma16<true, t * kTileRowBytes>(wbase, w_off[rg][u], my_lds + (rg * T + t) * kTileBytes + u * 1024);
             });
         };
+        constexpr std::integral_constant<int, 0> kZero{};
+        constexpr std::integral_constant<int, T> kAllTiles{};
+        constexpr std::integral_constant<int, kTilesBeforeX> kHead{};
+        constexpr std::integral_constant<int, T - kTilesBeforeX> kTail{};
 #pragma unroll
         for (int rg = 0; rg < kGroupsBeforeX; ++rg)
-            issue_w(rg);
+            issue_w(rg, kZero, kAllTiles);
+        if constexpr (kTilesBeforeX > 0)
+            issue_w(0, kZero, kHead);
 #pragma unroll
         for (int f = 0; f < FMX; ++f) {
             if constexpr (XDMA) {
@@ -279,9 +289,11 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
                 });
             }
         }
+        if constexpr (kTilesBeforeX > 0)
+            issue_w(0, kHead, kTail);
 #pragma unroll
-        for (int rg = kGroupsBeforeX; rg < R; ++rg)
-            issue_w(rg);
+        for (int rg = kGroupsBeforeX + (kTilesBeforeX > 0 ? 1 : 0); rg < R; ++rg)
+            issue_w(rg, kZero, kAllTiles);
     }
 
     // ---- one row group at a time
