@@ -180,12 +180,17 @@ __global__ __launch_bounds__(256) void fp6_convert_kernel(ConvertJob ja, Convert
 
 // ---- GEMM ---------------------------------------------------------------------------------
 
-__device__ __forceinline__ void dma16(const void *sbase, unsigned voff, unsigned lds_addr)
+// 16 bytes per lane from sbase + voff + IMM straight into LDS at place + ring + IMM + 16 * lane
+// (the hardware adds the instruction's constant on both sides, which is what a linear copy
+// wants; the two scalar summands of the LDS address are added on the way into M0).
+template <int IMM>
+__device__ __forceinline__ void dma16(const void *sbase, unsigned voff, unsigned place, unsigned ring)
 {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+    static_assert(IMM >= 0 && IMM < 4096, "13-bit signed immediate");
+    asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%4"
                  :
-                 : "v"(voff), "s"(sbase), "s"(lds_addr)
-                 : "memory");
+                 : "v"(voff), "s"(sbase), "s"(place), "s"(ring), "n"(IMM)
+                 : "memory", "scc");
 }
 
 // Marks a value as used at this point of the program without generating code.
@@ -253,11 +258,18 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
     const int total_stages = my_tiles * KT;
 
     // ---- load side: stage = 24 KiB of X fragments then 24 KiB of W fragments, copied
-    //      linearly; wave w moves the 1-KiB chunks w, w + NWAVES, ...
+    //      linearly; wave w moves CH/2 consecutive 1-KiB chunks of either half, so that the
+    //      chunks of a half differ only in the instruction's constant.
     const uint8_t *xptr = XW, *wptr = WW;  // wave-uniform: this tile's current stage
     int ld_it = 0, ld_k = 0, issued = 0;
     const unsigned lds_base = (unsigned)(size_t)I4L_LDS(lds);
     const unsigned lane16 = (unsigned)lane * 16u;
+    constexpr int kHalfChunks = C::CH / 2;
+    static_assert(kHalfChunks * 1024 <= 4096, "a wave's chunks of one half must be within reach of the constant");
+    const unsigned ld_voff = lane16 + (unsigned)(wave * kHalfChunks * 1024);
+    const unsigned place_x = lds_base + (unsigned)(wave * kHalfChunks * 1024);
+    const unsigned place_w = place_x + (unsigned)kOperandStageBytes;
+    unsigned wr_ring = 0;  // offset of the stage buffer being filled: (issued % kStages) * kStageBytes
 
     auto ld_setup_tile = [&](int it) {
         int tm, tn;
@@ -265,14 +277,16 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
         xptr = XW + (size_t)tm * KT * kOperandStageBytes;
         wptr = WW + (size_t)tn * KT * kOperandStageBytes;
     };
-    auto ld_chunk = [&](int c) {
-        const int q = c * C::NWAVES + wave;  // chunk of the stage, 0 .. CHUNKS-1
-        const bool is_x = q < C::CHUNKS / 2;
-        const uint8_t *src = is_x ? xptr + q * 1024 : wptr + (q - C::CHUNKS / 2) * 1024;
-        dma16(src, lane16, lds_base + (issued % kStages) * kStageBytes + q * 1024);
+    auto ld_chunk = [&](auto c) {  // c < CH/2: X half, else W half
+        constexpr int cc = decltype(c)::value;
+        if constexpr (cc < kHalfChunks)
+            dma16<cc * 1024>(xptr, ld_voff, place_x, wr_ring);
+        else
+            dma16<(cc - kHalfChunks) * 1024>(wptr, ld_voff, place_w, wr_ring);
     };
     auto ld_advance = [&]() {
         ++issued;
+        wr_ring = wr_ring + kStageBytes == kLdsBytes ? 0u : wr_ring + kStageBytes;
         ++ld_k;
         xptr += kOperandStageBytes;
         wptr += kOperandStageBytes;
@@ -295,16 +309,15 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
     // every iteration gs finishes stage gs+2 in its first unit and begins stage gs+3 in its
     // second, so the loop body needs no branch around a load.
     ld_setup_tile(0);
+    auto ld_chunks = [&]<int... CC>(std::integer_sequence<int, CC...>) {
+        (ld_chunk(std::integral_constant<int, CC>{}), ...);
+    };
 #pragma unroll
     for (int s = 0; s < kStages - 1; ++s) {
-#pragma unroll
-        for (int c = 0; c < C::CH; ++c)
-            ld_chunk(c);
+        ld_chunks(std::make_integer_sequence<int, C::CH>{});
         ld_advance();
     }
-#pragma unroll
-    for (int c = 0; c < C::CH / 2; ++c)
-        ld_chunk(c);
+    ld_chunks(std::make_integer_sequence<int, C::CH / 2>{});
 
     // ---- math side.  Unit u = (stage, k-fragment kf); its operands are FM X fragments
     //      and FN W fragments, each 6 VGPRs read as 16 + 8 bytes.  While the MFMAs of unit
@@ -320,8 +333,8 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
 
     // Read instruction r (0 .. 2*(FM+FN)-1) of unit (st, kf) into register set p:
     // fragment r/2, 16-byte part for even r, 8-byte part for odd r; X fragments first.
-    auto read_op = [&](int st, int kf, int p, int r) {
-        const uint8_t *base = lds + (st % kStages) * kStageBytes + kf * kFragsRows * kFragBytes;
+    auto read_op = [&](unsigned ring, int kf, int p, int r) {  // ring: offset of the stage's buffer
+        const uint8_t *base = lds + ring + kf * kFragsRows * kFragBytes;
         const int f = r >> 1;
         const bool is_x = f < C::FM;
         const int idx = is_x ? f : f - C::FM;
@@ -364,13 +377,13 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
     constexpr int kDmaFirstSlot = C::SLOTS / 2;
     static_assert(kReads <= kReadsPerSlot * C::SLOTS, "not enough slots for the LDS reads");
     static_assert(kDmaFirstSlot + C::CH / 2 <= C::SLOTS, "not enough slots for the loads");
-    auto spread = [&](auto slot_tag, int read_st, int read_kf, int read_p, int half_pos) {
+    auto spread = [&](auto slot_tag, unsigned read_ring, int read_kf, int read_p, auto half_pos) {
         constexpr int slot = decltype(slot_tag)::value;
 #pragma unroll
         for (int r = slot * kReadsPerSlot; r < (slot + 1) * kReadsPerSlot && r < kReads; ++r)
-            read_op(read_st, read_kf, read_p, r);
+            read_op(read_ring, read_kf, read_p, r);
         if constexpr (slot >= kDmaFirstSlot && slot < kDmaFirstSlot + C::CH / 2) {
-            ld_chunk(half_pos * (C::CH / 2) + slot - kDmaFirstSlot);
+            ld_chunk(std::integral_constant<int, decltype(half_pos)::value * (C::CH / 2) + slot - kDmaFirstSlot>{});
         }
     };
 
@@ -381,8 +394,10 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
     asm volatile("" ::: "memory");
 #pragma unroll
     for (int r = 0; r < kReads; ++r)
-        read_op(0, 0, 0, r);
+        read_op(0u, 0, 0, r);
 
+    unsigned rd_cur = 0, rd_next = kStageBytes;  // buffer offsets of stages gs and gs+1
+    int stores_behind = 0;  // a tile has just been stored: its stores sit behind the loads waited for next
 #pragma unroll 1
     for (int gs = 0; gs < total_stages; ++gs) {
         if (kk == 0) {
@@ -397,7 +412,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
 
         // ---- unit (gs, 0): reads unit (gs, 1); finishes the loads of stage gs+2
         unit(std::integral_constant<int, 0>{}, [&](auto slot_tag) {
-            spread(slot_tag, gs, 1, 1, 1);
+            spread(slot_tag, rd_cur, 1, 1, std::integral_constant<int, 1>{});
             if constexpr (decltype(slot_tag)::value == C::SLOTS - 1)
                 ld_advance();
         });
@@ -408,9 +423,10 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
         //      normally one younger stage (gs+2) is in flight behind it, and in the first
         //      stage after a tile end that tile's C stores sit behind it as well.
         {
-            if (cur_it > 0 && kk < 1) {
+            if (stores_behind) {
                 constexpr int with_stores = C::CH + C::STORES;
                 __builtin_amdgcn_s_waitcnt(I4L_WAIT_VM_LGKM0(with_stores < 63 ? with_stores : 63));
+                stores_behind = 0;
             } else {
                 __builtin_amdgcn_s_waitcnt(I4L_WAIT_VM_LGKM0(C::CH));
             }
@@ -421,7 +437,11 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
         // ---- unit (gs, 1): reads unit (gs+1, 0) (a stale buffer past the last stage, never
         //      multiplied into a stored tile); begins the loads of stage gs+3 into the
         //      buffer of stage gs
-        unit(std::integral_constant<int, 1>{}, [&](auto slot_tag) { spread(slot_tag, gs + 1, 0, 0, 0); });
+        unit(std::integral_constant<int, 1>{}, [&](auto slot_tag) {
+            spread(slot_tag, rd_next, 0, 0, std::integral_constant<int, 0>{});
+        });
+        rd_cur = rd_next;
+        rd_next = rd_next + kStageBytes == kLdsBytes ? 0u : rd_next + kStageBytes;
         ++kk;
         if (kk == KT) {
             // ---- store the tile.  X is the MFMA A operand: accumulator t of tile (i, j) is
@@ -498,6 +518,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
             }
             kk = 0;
             ++cur_it;
+            stores_behind = 1;
         }
     }
 }
