@@ -277,12 +277,12 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
         xptr = XW + (size_t)tm * KT * kOperandStageBytes;
         wptr = WW + (size_t)tn * KT * kOperandStageBytes;
     };
-    auto ld_chunk = [&](auto c) {  // c < CH/2: X half, else W half
+    auto ld_chunk = [&](auto c, unsigned ring) {  // c < CH/2: X half, else W half; ring: the buffer's offset
         constexpr int cc = decltype(c)::value;
         if constexpr (cc < kHalfChunks)
-            dma16<cc * 1024>(xptr, ld_voff, place_x, wr_ring);
+            dma16<cc * 1024>(xptr, ld_voff, place_x, ring);
         else
-            dma16<(cc - kHalfChunks) * 1024>(wptr, ld_voff, place_w, wr_ring);
+            dma16<(cc - kHalfChunks) * 1024>(wptr, ld_voff, place_w, ring);
     };
     auto ld_advance = [&]() {
         ++issued;
@@ -310,7 +310,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
     // second, so the loop body needs no branch around a load.
     ld_setup_tile(0);
     auto ld_chunks = [&]<int... CC>(std::integer_sequence<int, CC...>) {
-        (ld_chunk(std::integral_constant<int, CC>{}), ...);
+        (ld_chunk(std::integral_constant<int, CC>{}, wr_ring), ...);
     };
 #pragma unroll
     for (int s = 0; s < kStages - 1; ++s) {
@@ -377,13 +377,13 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
     constexpr int kDmaFirstSlot = C::SLOTS / 2;
     static_assert(kReads <= kReadsPerSlot * C::SLOTS, "not enough slots for the LDS reads");
     static_assert(kDmaFirstSlot + C::CH / 2 <= C::SLOTS, "not enough slots for the loads");
-    auto spread = [&](auto slot_tag, unsigned read_ring, int read_kf, int read_p, auto half_pos) {
+    auto spread = [&](auto slot_tag, unsigned read_ring, int read_kf, int read_p, auto half_pos, unsigned load_ring) {
         constexpr int slot = decltype(slot_tag)::value;
 #pragma unroll
         for (int r = slot * kReadsPerSlot; r < (slot + 1) * kReadsPerSlot && r < kReads; ++r)
             read_op(read_ring, read_kf, read_p, r);
         if constexpr (slot >= kDmaFirstSlot && slot < kDmaFirstSlot + C::CH / 2) {
-            ld_chunk(std::integral_constant<int, decltype(half_pos)::value * (C::CH / 2) + slot - kDmaFirstSlot>{});
+            ld_chunk(std::integral_constant<int, decltype(half_pos)::value * (C::CH / 2) + slot - kDmaFirstSlot>{}, load_ring);
         }
     };
 
@@ -396,10 +396,15 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
     for (int r = 0; r < kReads; ++r)
         read_op(0u, 0, 0, r);
 
-    unsigned rd_cur = 0, rd_next = kStageBytes;  // buffer offsets of stages gs and gs+1
     int stores_behind = 0;  // a tile has just been stored: its stores sit behind the loads waited for next
-#pragma unroll 1
-    for (int gs = 0; gs < total_stages; ++gs) {
+    // One iteration of the stage loop, for the stage whose buffer is ring position RING.  The
+    // loop below is unrolled over the three positions, so that every LDS address is a
+    // loop-invariant register plus a constant and every buffer offset a constant.
+    auto iteration = [&](auto ring_tag) {
+        constexpr unsigned rd_cur = decltype(ring_tag)::value * kStageBytes;              // stage gs
+        constexpr unsigned rd_next = (decltype(ring_tag)::value + 1) % kStages * kStageBytes;  // stage gs+1
+        constexpr unsigned wr_first = (decltype(ring_tag)::value + 2) % kStages * kStageBytes; // stage gs+2
+        constexpr unsigned wr_second = rd_cur;                                            // stage gs+3
         if (kk == 0) {
 #pragma unroll
             for (int i = 0; i < C::FN; ++i)
@@ -412,7 +417,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
 
         // ---- unit (gs, 0): reads unit (gs, 1); finishes the loads of stage gs+2
         unit(std::integral_constant<int, 0>{}, [&](auto slot_tag) {
-            spread(slot_tag, rd_cur, 1, 1, std::integral_constant<int, 1>{});
+            spread(slot_tag, rd_cur, 1, 1, std::integral_constant<int, 1>{}, wr_first);
             if constexpr (decltype(slot_tag)::value == C::SLOTS - 1)
                 ld_advance();
         });
@@ -438,10 +443,8 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
         //      multiplied into a stored tile); begins the loads of stage gs+3 into the
         //      buffer of stage gs
         unit(std::integral_constant<int, 1>{}, [&](auto slot_tag) {
-            spread(slot_tag, rd_next, 0, 0, std::integral_constant<int, 0>{});
+            spread(slot_tag, rd_next, 0, 0, std::integral_constant<int, 0>{}, wr_second);
         });
-        rd_cur = rd_next;
-        rd_next = rd_next + kStageBytes == kLdsBytes ? 0u : rd_next + kStageBytes;
         ++kk;
         if (kk == KT) {
             // ---- store the tile.  X is the MFMA A operand: accumulator t of tile (i, j) is
@@ -520,6 +523,17 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
             ++cur_it;
             stores_behind = 1;
         }
+    };
+    for (int gs = 0;;) {
+        iteration(std::integral_constant<int, 0>{});
+        if (++gs == total_stages)
+            break;
+        iteration(std::integral_constant<int, 1>{});
+        if (++gs == total_stages)
+            break;
+        iteration(std::integral_constant<int, 2>{});
+        if (++gs == total_stages)
+            break;
     }
 }
 
