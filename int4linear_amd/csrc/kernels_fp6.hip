@@ -43,7 +43,7 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 // s_waitcnt immediate for gfx9: vmcnt[3:0] bits 3:0, vmcnt[5:4] bits 15:14, expcnt bits
 // 6:4, lgkmcnt bits 11:8.  VM only leaves the others at "no wait".
 #define I4L_WAIT_VM(n) ((0x0F70) | ((n) & 0xF) | ((((n) >> 4) & 0x3) << 14))
-#define I4L_WAIT_VM_LGKM0(n) ((0x0070) | ((n) & 0xF) | ((((n) >> 4) & 0x3) << 14))
+#define I4L_WAIT_LGKM0 0xC07F
 
 constexpr int kTileRows = 256;                        // rows of either operand per tile
 constexpr int kFragRows = 32;                         // rows of one MFMA operand
@@ -57,6 +57,12 @@ constexpr int kOperandStageBytes = kFragsK * kFragsRows * kFragBytes;  // 24 KiB
 constexpr int kStageBytes = 2 * kOperandStageBytes;                    // 48 KiB
 constexpr int kStages = 3;
 constexpr int kLdsBytes = kStages * kStageBytes;                       // 144 KiB
+constexpr int kStaggerGroups = 8;                     // start groups within an XCD (power of two)
+#ifndef FP6_STAGGER_TICKS
+#define FP6_STAGGER_TICKS 80
+#endif
+constexpr int kStaggerTicks = FP6_STAGGER_TICKS;      // delay between groups, in 10-ns ticks of the constant clock
+constexpr int kStaggerMinRounds = 3;                  // tiles per workgroup from which the start is staggered
 constexpr int kScale = 127 + 3;                       // E8M0 block scale 2^3 for both operands
 
 // ---- converter --------------------------------------------------------------------------
@@ -255,7 +261,18 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
     if (bid >= total_tiles)
         return;
     const int my_tiles = (total_tiles - bid + nblk - 1) / nblk;
-    const int total_stages = my_tiles * KT;
+    // Workgroups that start together reach every tile end together, and the stores of all
+    // tiles then queue for the same path to memory while no CU computes.  With three or
+    // more tiles per workgroup the 32 workgroups of an XCD (ids congruent mod 8) therefore
+    // start in eight groups a fraction of a microsecond apart: their tile ends stay that
+    // far apart for the rest of the launch, which costs the spread once at the end and
+    // saves most of the wait at every tile end before.
+    if (total_tiles >= kStaggerMinRounds * nblk) {
+        const int grp = (bid >> 3) & (kStaggerGroups - 1);
+        const unsigned long long until = wall_clock64() + (unsigned long long)(grp * kStaggerTicks);
+        while (wall_clock64() < until)
+            __builtin_amdgcn_s_sleep(2);
+    }
 
     // ---- load side: stage = 24 KiB of X fragments then 24 KiB of W fragments, copied
     //      linearly; wave w moves CH/2 consecutive 1-KiB chunks of either half, so that the
@@ -400,21 +417,23 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
     // One iteration of the stage loop, for the stage whose buffer is ring position RING.  The
     // loop below is unrolled over the three positions, so that every LDS address is a
     // loop-invariant register plus a constant and every buffer offset a constant.
-    auto iteration = [&](auto ring_tag) {
+    auto clear_acc = [&]() {
+#pragma unroll
+        for (int i = 0; i < C::FN; ++i)
+#pragma unroll
+            for (int j = 0; j < C::FM; ++j)
+#pragma unroll
+                for (int t = 0; t < 16; ++t)
+                    acc[i][j][t] = 0.f;
+    };
+    clear_acc();
+    // Returns true after the block's last tile.  Whatever a stage does only at a tile's end
+    // (store, clear the accumulators, test for the end) sits behind the one branch on kk.
+    auto iteration = [&](auto ring_tag) -> bool {
         constexpr unsigned rd_cur = decltype(ring_tag)::value * kStageBytes;              // stage gs
         constexpr unsigned rd_next = (decltype(ring_tag)::value + 1) % kStages * kStageBytes;  // stage gs+1
         constexpr unsigned wr_first = (decltype(ring_tag)::value + 2) % kStages * kStageBytes; // stage gs+2
         constexpr unsigned wr_second = rd_cur;                                            // stage gs+3
-        if (kk == 0) {
-#pragma unroll
-            for (int i = 0; i < C::FN; ++i)
-#pragma unroll
-                for (int j = 0; j < C::FM; ++j)
-#pragma unroll
-                    for (int t = 0; t < 16; ++t)
-                        acc[i][j][t] = 0.f;
-        }
-
         // ---- unit (gs, 0): reads unit (gs, 1); finishes the loads of stage gs+2
         unit(std::integral_constant<int, 0>{}, [&](auto slot_tag) {
             spread(slot_tag, rd_cur, 1, 1, std::integral_constant<int, 1>{}, wr_first);
@@ -424,17 +443,23 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
 
         // ---- between the units: every LDS read of stage gs has been issued; once they
         //      have returned (lgkmcnt 0) and every wave is here, the buffer of stage gs is
-        //      free for stage gs+3.  Stage gs+1 must have landed: loads complete in order,
-        //      normally one younger stage (gs+2) is in flight behind it, and in the first
-        //      stage after a tile end that tile's C stores sit behind it as well.
+        //      free for stage gs+3.  Stage gs+1 must have landed: memory operations complete
+        //      in order and normally one younger stage (gs+2) is in flight behind it.  In
+        //      the first stage after a tile end that tile's C stores sit behind it as well:
+        //      they are more than the counter can hold (63), so their issue has already
+        //      waited for everything older, and no wait is wanted (one for CH would stall
+        //      until the stores have drained).  The common case falls through the branch.
         {
-            if (stores_behind) {
-                constexpr int with_stores = C::CH + C::STORES;
-                __builtin_amdgcn_s_waitcnt(I4L_WAIT_VM_LGKM0(with_stores < 63 ? with_stores : 63));
-                stores_behind = 0;
-            } else {
-                __builtin_amdgcn_s_waitcnt(I4L_WAIT_VM_LGKM0(C::CH));
-            }
+            static_assert(C::STORES >= 64, "the stores of a tile must saturate the counter");
+            asm volatile("s_cmp_lg_u32 %0, 0\n\t"
+                         "s_cbranch_scc1 1f\n\t"
+                         "s_waitcnt vmcnt(%1)\n"
+                         "1:"
+                         :
+                         : "s"(stores_behind), "n"(C::CH)
+                         : "scc", "memory");
+            stores_behind = 0;
+            __builtin_amdgcn_s_waitcnt(I4L_WAIT_LGKM0);
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
         }
@@ -446,7 +471,9 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
             spread(slot_tag, rd_next, 0, 0, std::integral_constant<int, 0>{}, wr_second);
         });
         ++kk;
-        if (kk == KT) {
+        if (kk != KT)
+            return false;
+        {
             // ---- store the tile.  X is the MFMA A operand: accumulator t of tile (i, j) is
             //   m = 32*j + 8*(t/4) + 4*(lane/32) + t%4,  n = 32*i + lane%32,
             // so one dword store writes two rows of 32 consecutive n (128 B each).
@@ -522,17 +549,16 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
             kk = 0;
             ++cur_it;
             stores_behind = 1;
+            clear_acc();
         }
+        return cur_it == my_tiles;
     };
-    for (int gs = 0;;) {
-        iteration(std::integral_constant<int, 0>{});
-        if (++gs == total_stages)
+    for (;;) {
+        if (iteration(std::integral_constant<int, 0>{}))
             break;
-        iteration(std::integral_constant<int, 1>{});
-        if (++gs == total_stages)
+        if (iteration(std::integral_constant<int, 1>{}))
             break;
-        iteration(std::integral_constant<int, 2>{});
-        if (++gs == total_stages)
+        if (iteration(std::integral_constant<int, 2>{}))
             break;
     }
 }
