@@ -58,11 +58,8 @@ constexpr int kStageBytes = 2 * kOperandStageBytes;                    // 48 KiB
 constexpr int kStages = 3;
 constexpr int kLdsBytes = kStages * kStageBytes;                       // 144 KiB
 constexpr int kStaggerGroups = 8;                     // start groups within an XCD (power of two)
-#ifndef FP6_STAGGER_TICKS
-#define FP6_STAGGER_TICKS 80
-#endif
-constexpr int kStaggerTicks = FP6_STAGGER_TICKS;      // delay between groups, in 10-ns ticks of the constant clock
-constexpr int kStaggerMinRounds = 3;                  // tiles per workgroup from which the start is staggered
+constexpr int kStaggerTicks = 120;                    // delay between groups, in 10-ns ticks of the constant clock
+constexpr int kStaggerMinRounds = 2;                  // tiles per workgroup from which the start is staggered
 constexpr int kScale = 127 + 3;                       // E8M0 block scale 2^3 for both operands
 
 // ---- converter --------------------------------------------------------------------------
@@ -262,9 +259,9 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
         return;
     const int my_tiles = (total_tiles - bid + nblk - 1) / nblk;
     // Workgroups that start together reach every tile end together, and the stores of all
-    // tiles then queue for the same path to memory while no CU computes.  With three or
+    // tiles then queue for the same path to memory while no CU computes.  With two or
     // more tiles per workgroup the 32 workgroups of an XCD (ids congruent mod 8) therefore
-    // start in eight groups a fraction of a microsecond apart: their tile ends stay that
+    // start in eight groups about a microsecond apart: their tile ends stay that
     // far apart for the rest of the launch, which costs the spread once at the end and
     // saves most of the wait at every tile end before.
     if (total_tiles >= kStaggerMinRounds * nblk) {
