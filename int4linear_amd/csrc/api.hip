@@ -85,14 +85,15 @@ bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 
 // The FP6 path pays off once its 256 x 256 tiles can occupy a good part of the device and K
 // is long enough to amortise the converter pass (a fixed cost of about (M + N) * K * 1.25
-// bytes of HBM traffic).  Measured crossovers against the int8 kernel: 128 tiles at K = 4096
-// and 256 tiles at K = 1024 still favour int8; 144 tiles at K = 3072, 256 tiles at K = 2048
-// and 1024 tiles at any K favour FP6.
+// bytes of HBM traffic).  Measured against the int8 kernel (tiles, K -> faster kernel):
+// 128, 4096 -> tie; 128, 14336 -> FP6 by 20 %; 144, 3072 -> FP6; 256, 2048 -> int8 by 5 %;
+// 512, 2048 -> FP6 by 20 %; 512, 1024 -> FP6 by 3 %; 1024, 1024 -> tie; 1024, 512 -> int8
+// by 10 %.
 bool fp6_worthwhile(int m, int n, int k)
 {
     const long tiles = (long)((m + 255) / 256) * ((n + 255) / 256);
-    return fp6_supports(m, n, k) && tiles >= 144 && (k >= 2048 || tiles >= 1024) &&
-           fp6_workspace_bytes(m, n, k) <= g_workspace_limit.load();
+    const bool pays = (tiles >= 128 && k >= 8192) || (tiles >= 144 && k >= 3072) || (tiles >= 384 && k >= 1024);
+    return pays && fp6_supports(m, n, k) && fp6_workspace_bytes(m, n, k) <= g_workspace_limit.load();
 }
 
 // K that is not a multiple of 128 fits neither the int8 nor the weight-streaming kernel,
