@@ -275,7 +275,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
     //      linearly; wave w moves CH/2 consecutive 1-KiB chunks of either half, so that the
     //      chunks of a half differ only in the instruction's constant.
     const uint8_t *xptr = XW, *wptr = WW;  // wave-uniform: this tile's current stage
-    int ld_it = 0, ld_k = 0, issued = 0;
+    int ld_it = 0, ld_k = 0;
     const unsigned lds_base = (unsigned)(size_t)I4L_LDS(lds);
     const unsigned lane16 = (unsigned)lane * 16u;
     constexpr int kHalfChunks = C::CH / 2;
@@ -283,7 +283,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
     const unsigned ld_voff = lane16 + (unsigned)(wave * kHalfChunks * 1024);
     const unsigned place_x = lds_base + (unsigned)(wave * kHalfChunks * 1024);
     const unsigned place_w = place_x + (unsigned)kOperandStageBytes;
-    unsigned wr_ring = 0;  // offset of the stage buffer being filled: (issued % kStages) * kStageBytes
+    unsigned wr_ring = 0;  // the prologue's: offset of the stage buffer being filled
 
     auto ld_setup_tile = [&](int it) {
         int tm, tn;
@@ -299,7 +299,6 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
             dma16<(cc - kHalfChunks) * 1024>(wptr, ld_voff, place_w, ring);
     };
     auto ld_advance = [&]() {
-        ++issued;
         wr_ring = wr_ring + kStageBytes == kLdsBytes ? 0u : wr_ring + kStageBytes;
         ++ld_k;
         xptr += kOperandStageBytes;
