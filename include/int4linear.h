@@ -15,8 +15,8 @@
  *
  * All pointers named *_d are device pointers owned by the caller.  The only device
  * memory the library itself allocates is one workspace per device (see
- * int4linear_workspace_bytes), which holds the FP6 kernel's converted operands or the
- * partial sums of the int8 kernel's split-K form: created on first need, grown when a
+ * int4linear_workspace_bytes), which holds the FP6 kernel's converted operands and the
+ * partial sums of either MFMA kernel's split-K form: created on first need, grown when a
  * larger problem arrives, never larger than the workspace limit, freed by
  * int4linear_release_workspace or at process exit.  With the limit set to 0 no entry
  * point allocates anything.
@@ -111,8 +111,9 @@ int int4linear_gemm_fp6_converted(const void *a_conv_d, const void *b_conv_d, vo
                                   int m, int n, int k, void *stream);
 
 /* Bytes of internal workspace INT4LINEAR_KERNEL_AUTO would use for a shape on the current
- * device (0 when the chosen kernel needs none, and for the split-K form before the
- * device's first call). */
+ * device (0 when the chosen kernel needs none; the split-K forms depend on the device's CU
+ * count, so before the device's first call the int8 form reports 0 and the FP6 form the
+ * converted operands alone). */
 size_t int4linear_workspace_bytes(int m, int n, int k);
 
 /* Upper bound for the internal workspace (default 1 GiB).  Shapes that would need more,

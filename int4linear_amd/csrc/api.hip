@@ -86,23 +86,26 @@ bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 // The FP6 path pays off once its 256 x 256 tiles can occupy a good part of the device and K
 // is long enough to amortise the converter pass (a fixed cost of about (M + N) * K * 1.25
 // bytes of HBM traffic).  Measured against the int8 kernel (tiles, K -> faster kernel):
-// 128, 4096 -> tie; 128, 14336 -> FP6 by 20 %; 144, 3072 -> FP6; 256, 2048 -> int8 by 5 %;
-// 512, 2048 -> FP6 by 20 %; 512, 1024 -> FP6 by 3 %; 1024, 1024 -> tie; 1024, 512 -> int8
-// by 10 %.
-bool fp6_worthwhile(int m, int n, int k)
+// 128, 4096 -> tie; 128, 8192 -> FP6 by 8 %; 128, 14336 -> FP6 by 20 %; 144, 3072 -> FP6;
+// 256, 2048 -> int8 by 5 %; 512, 2048 -> FP6 by 20 %; 512, 1024 -> FP6 by 3 %; 1024, 1024
+// -> tie; 1024, 512 -> int8 by 10 %.  Split over K (64 tiles or fewer on 256 CUs): 64 tiles
+// at K = 14336 -> FP6 by 9 %, at K = 28672 by 16 %; 48 tiles at K = 8192 and 32 or fewer
+// at K = 14336 -> int8 (itself split over K).
+bool fp6_worthwhile(int m, int n, int k, const DeviceInfo &dev)
 {
     const long tiles = (long)((m + 255) / 256) * ((n + 255) / 256);
-    const bool pays = (tiles >= 128 && k >= 8192) || (tiles >= 144 && k >= 3072) || (tiles >= 384 && k >= 1024);
-    return pays && fp6_supports(m, n, k) && fp6_workspace_bytes(m, n, k) <= g_workspace_limit.load();
+    const bool pays = (tiles >= 128 && k >= 8192) || (tiles >= 144 && k >= 3072) || (tiles >= 384 && k >= 1024) ||
+                      (tiles >= 64 && k >= 12288 && fp6_ksplit(m, n, k, dev) > 1);
+    return pays && fp6_supports(m, n, k) && fp6_workspace_bytes(m, n, k, dev) <= g_workspace_limit.load();
 }
 
 // K that is not a multiple of 128 fits neither the int8 nor the weight-streaming kernel,
 // but the FP6 converter pads K with zeros: beyond a few million multiply-adds that beats
 // the scalar kernel by orders of magnitude even for a handful of rows.
-bool fp6_for_ragged_k(int m, int n, int k)
+bool fp6_for_ragged_k(int m, int n, int k, const DeviceInfo &dev)
 {
     return (k % 128) != 0 && fp6_supports(m, n, k) && (double)m * n * k >= (double)(1 << 22) &&
-           fp6_workspace_bytes(m, n, k) <= g_workspace_limit.load();
+           fp6_workspace_bytes(m, n, k, dev) <= g_workspace_limit.load();
 }
 
 // What is known of the current device: all zero before the first call on it.
@@ -120,11 +123,11 @@ int pick_kernel(int m, int n, int k, const DeviceInfo &dev)
 {
     if (skinny_preferred(m, n, k, dev))
         return INT4LINEAR_KERNEL_SKINNY;
-    if (fp6_worthwhile(m, n, k))
+    if (fp6_worthwhile(m, n, k, dev))
         return INT4LINEAR_KERNEL_FP6;
     if (mfma_supports(m, n, k))
         return INT4LINEAR_KERNEL_MFMA;
-    if (fp6_for_ragged_k(m, n, k))
+    if (fp6_for_ragged_k(m, n, k, dev))
         return INT4LINEAR_KERNEL_FP6;
     return INT4LINEAR_KERNEL_SIMPLE;
 }
@@ -188,7 +191,7 @@ int run_fp6(PerDevice *pd, const void *a, const void *b, void *c, int m, int n, 
 {
     std::lock_guard<std::mutex> lock(pd->ws_mutex);
     void *ws = nullptr;
-    const int st = acquire_workspace(pd, fp6_workspace_bytes(m, n, k), stream, &ws);
+    const int st = acquire_workspace(pd, fp6_workspace_bytes(m, n, k, pd->info), stream, &ws);
     if (st != INT4LINEAR_OK)
         return st;
     const hipError_t e = launch_fp6(a, b, c, m, n, k, ws, ep, pd->info, stream);
@@ -467,7 +470,7 @@ size_t int4linear_workspace_bytes(int m, int n, int k)
     const DeviceInfo info = current_device_info();
     const int kernel = pick_kernel(m, n, k, info);
     if (kernel == INT4LINEAR_KERNEL_FP6)
-        return fp6_workspace_bytes(m, n, k);
+        return fp6_workspace_bytes(m, n, k, info);
     if (kernel == INT4LINEAR_KERNEL_MFMA) {
         // the split-K form needs the device's CU count: 0 before the first call on a device
         if (info.cu_count == 0)
@@ -521,7 +524,7 @@ int version_kernel(int version, int m, int n, int k)
     case 21:
         return INT4LINEAR_KERNEL_AUTO;
     case 20:
-        if (fp6_supports(m, n, k) && fp6_workspace_bytes(m, n, k) <= g_workspace_limit.load() &&
+        if (fp6_supports(m, n, k) && fp6_workspace_bytes(m, n, k, current_device_info()) <= g_workspace_limit.load() &&
             !skinny_preferred(m, n, k, current_device_info()))
             return INT4LINEAR_KERNEL_FP6;
         [[fallthrough]];

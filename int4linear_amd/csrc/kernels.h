@@ -59,9 +59,13 @@ hipError_t launch_mfma_tile(const void *a, const void *b, void *c, int m, int n,
                             const Epilogue &ep, const DeviceInfo &dev, hipStream_t stream);
 
 // FP6-MFMA path: converts both operands into a workspace of fp6_workspace_bytes() bytes
-// (256-byte aligned), then runs the GEMM on it.  Requires K % 128 == 0, K < 2^18.
+// (256-byte aligned), then runs the GEMM on it.  Requires K % 8 == 0, K < 2^18.  With few
+// output tiles and long K the GEMM is split over K (fp6_ksplit() slices per tile, 1 = not
+// split; it depends on the device's CU count and is 1 while that is unknown): the partial
+// sums go into slabs in the same workspace and a second kernel adds them up.
 bool fp6_supports(int m, int n, int k);
-size_t fp6_workspace_bytes(int m, int n, int k);
+int fp6_ksplit(int m, int n, int k, const DeviceInfo &dev);
+size_t fp6_workspace_bytes(int m, int n, int k, const DeviceInfo &dev);
 hipError_t fp6_init(const DeviceInfo &dev);
 // The two halves of launch_fp6 on caller-owned buffers: an operand of `rows` rows converts
 // into fp6_operand_bytes(rows, k) bytes (256-byte aligned); the GEMM runs on two of those.

@@ -242,7 +242,7 @@ struct Fp6Config {
 template <class C>
 __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
     const uint8_t *__restrict__ XW, const uint8_t *__restrict__ WW, int32_t *__restrict__ Y,
-    int M, int N, int K, int tiles_m, int tiles_n, Epilogue ep)
+    int M, int N, int K, int tiles_m, int tiles_n, int ksplit, Epilogue ep)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
@@ -250,11 +250,17 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wm = wave / C::WAVES_N;
     const int wn = wave % C::WAVES_N;
-    const int KT = K / kStageK;
-    const int total_tiles = tiles_m * tiles_n;
+    // With ksplit > 1 a work item is one K-slice of one tile: item v is slice v / tiles of
+    // tile v % tiles (so the items of one slice are laid out like the tiles of an unsplit
+    // launch), covers KT of the KT_all stages, and stores its plain partial sums into slab
+    // `slice` of Y (M * N int32 each), which a second kernel adds up.
+    const int KT_all = K / kStageK;
+    const int KT = KT_all / ksplit;
+    const int tiles = tiles_m * tiles_n;
+    const int total_tiles = tiles * ksplit;  // work items
     const int nblk = gridDim.x;
     const int bid = blockIdx.x;
-    const bool ep_plain = !ep.bias && !ep.row_scale && !ep.col_scale && !ep.f32;
+    const bool ep_plain = ksplit > 1 || (!ep.bias && !ep.row_scale && !ep.col_scale && !ep.f32);
     if (bid >= total_tiles)
         return;
     const int my_tiles = (total_tiles - bid + nblk - 1) / nblk;
@@ -287,9 +293,11 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
 
     auto ld_setup_tile = [&](int it) {
         int tm, tn;
-        tile_coords(bid + it * nblk, total_tiles, tiles_m, tiles_n, tm, tn);
-        xptr = XW + (size_t)tm * KT * kOperandStageBytes;
-        wptr = WW + (size_t)tn * KT * kOperandStageBytes;
+        const int item = bid + it * nblk;
+        const int slice = item / tiles;
+        tile_coords(item - slice * tiles, tiles, tiles_m, tiles_n, tm, tn);
+        xptr = XW + ((size_t)tm * KT_all + (size_t)slice * KT) * kOperandStageBytes;
+        wptr = WW + ((size_t)tn * KT_all + (size_t)slice * KT) * kOperandStageBytes;
     };
     auto ld_chunk = [&](auto c, unsigned ring) {  // c < CH/2: X half, else W half; ring: the buffer's offset
         constexpr int cc = decltype(c)::value;
@@ -474,11 +482,13 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
             //   m = 32*j + 8*(t/4) + 4*(lane/32) + t%4,  n = 32*i + lane%32,
             // so one dword store writes two rows of 32 consecutive n (128 B each).
             int tm, tn;
-            tile_coords(bid + cur_it * nblk, total_tiles, tiles_m, tiles_n, tm, tn);
+            const int item = bid + cur_it * nblk;
+            const int slice = item / tiles;
+            tile_coords(item - slice * tiles, tiles, tiles_m, tiles_n, tm, tn);
             const int m0 = tm * kTileRows, n0 = tn * kTileRows;
             const int rows_left = M - m0;  // > 0
             const int cols_left = N - n0;  // > 0
-            int32_t *ybase = Y + (size_t)m0 * N + n0;
+            int32_t *ybase = Y + (size_t)slice * (size_t)M * (size_t)N + (size_t)m0 * N + n0;
             const size_t slab_rows = rows_left < kTileRows ? rows_left : kTileRows;
             const size_t extent = ((slab_rows - 1) * (size_t)N + (size_t)(cols_left < kTileRows ? cols_left : kTileRows)) * 4u;
             __amdgpu_buffer_rsrc_t rsrc =
@@ -577,9 +587,25 @@ bool fp6_supports(int m, int n, int k)
     return m >= 1 && n >= 1 && k >= 8 && k % 8 == 0 && k <= (1 << 18) - kStageK;
 }
 
-size_t fp6_workspace_bytes(int m, int n, int k)
+int fp6_ksplit(int m, int n, int k, const DeviceInfo &dev)
 {
-    return operand_ws_bytes(m, k) + operand_ws_bytes(n, k);
+    const long tiles = (long)((m + kTileRows - 1) / kTileRows) * ((n + kTileRows - 1) / kTileRows);
+    const int stages = (k + kStageK - 1) / kStageK;
+    // Measured: two slices of 128 tiles gain nothing over 128 unsplit tiles (the second kernel
+    // and the slabs cost what the idle half of the device did); four of 64 tiles gain 9-16 %.
+    if (dev.cu_count <= 0 || tiles * 4 > dev.cu_count)
+        return 1;
+    // The most slices that still leave a workgroup per CU, 2048 k per slice and equal slices.
+    for (int ks : {8, 7, 6, 5, 4, 3, 2})
+        if (tiles * ks <= dev.cu_count && stages % ks == 0 && stages / ks >= 16)
+            return ks;
+    return 1;
+}
+
+size_t fp6_workspace_bytes(int m, int n, int k, const DeviceInfo &dev)
+{
+    const int ks = fp6_ksplit(m, n, k, dev);
+    return operand_ws_bytes(m, k) + operand_ws_bytes(n, k) + (ks > 1 ? (size_t)ks * (size_t)m * (size_t)n * 4u : 0);
 }
 
 hipError_t fp6_init(const DeviceInfo &dev)
@@ -625,21 +651,67 @@ hipError_t launch_fp6_convert(const void *src, void *dst, int rows, int k, hipSt
     return launch_convert_jobs(make_job(src, dst, rows), ConvertJob{nullptr, nullptr, 0, 0}, k, stream);
 }
 
-hipError_t launch_fp6_gemm(const void *a_conv, const void *b_conv, void *c, int m, int n, int k,
-                           const Epilogue &ep, const DeviceInfo &dev, hipStream_t stream)
+namespace {
+
+// ksplit > 1: `c` is ksplit slabs of m * n partial sums and `ep` must be empty.
+hipError_t launch_gemm_items(const void *a_conv, const void *b_conv, void *c, int m, int n, int k, int ksplit,
+                             const Epilogue &ep, const DeviceInfo &dev, hipStream_t stream)
 {
     using C = Fp6Cfg;
     const int tiles_m = (m + kTileRows - 1) / kTileRows;
     const int tiles_n = (n + kTileRows - 1) / kTileRows;
-    const long total = (long)tiles_m * tiles_n;
+    const long total = (long)tiles_m * tiles_n * ksplit;
     if (total > 0x7fffffffL || (size_t)kTileRows * (size_t)n * 4u > 0x40000000ull)
         return hipErrorInvalidValue;
     long grid = (long)dev.cu_count * C::OCC;
     if (grid > total)
         grid = total;
     fp6_gemm_kernel<C><<<(unsigned)grid, C::THREADS, kLdsBytes, stream>>>(
-        (const uint8_t *)a_conv, (const uint8_t *)b_conv, (int32_t *)c, m, n, padded_k(k), tiles_m, tiles_n, ep);
+        (const uint8_t *)a_conv, (const uint8_t *)b_conv, (int32_t *)c, m, n, padded_k(k), tiles_m, tiles_n, ksplit, ep);
     return hipGetLastError();
+}
+
+// Second kernel of the split-K form: Y = epilogue(sum of the ksplit slabs), four outputs of
+// one row per thread (VEC: n % 4 == 0) or one.
+template <bool VEC>
+__global__ __launch_bounds__(256) void fp6_splitk_reduce_kernel(const int32_t *__restrict__ partial,
+                                                                int32_t *__restrict__ Y, size_t count, int ksplit,
+                                                                int N, Epilogue ep)
+{
+    constexpr int kPer = VEC ? 4 : 1;
+    const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * kPer;
+    if (i >= count)
+        return;
+    int sum[kPer] = {};
+    for (int s = 0; s < ksplit; ++s) {
+        const int32_t *src = partial + (size_t)s * count + i;
+        if constexpr (VEC) {
+            const v4i v = __builtin_nontemporal_load((const v4i *)src);
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                sum[q] += v[q];
+        } else {
+            sum[0] += *src;
+        }
+    }
+    const size_t row = i / (size_t)N;
+    const int col = (int)(i - row * (size_t)N);
+    const float rs = ep.row_scale ? ep.row_scale[row] : 1.f;
+#pragma unroll
+    for (int q = 0; q < kPer; ++q)
+        sum[q] = epilogue_value(ep, sum[q], ep.bias ? ep.bias[col + q] : 0, rs, ep.col_scale ? ep.col_scale[col + q] : 1.f);
+    if constexpr (VEC)
+        *(v4i *)(Y + i) = (v4i){sum[0], sum[1], sum[2], sum[3]};
+    else
+        Y[i] = sum[0];
+}
+
+}  // namespace
+
+hipError_t launch_fp6_gemm(const void *a_conv, const void *b_conv, void *c, int m, int n, int k,
+                           const Epilogue &ep, const DeviceInfo &dev, hipStream_t stream)
+{
+    return launch_gemm_items(a_conv, b_conv, c, m, n, k, 1, ep, dev, stream);
 }
 
 hipError_t launch_fp6(const void *a, const void *b, void *c, int m, int n, int k, void *workspace,
@@ -648,9 +720,23 @@ hipError_t launch_fp6(const void *a, const void *b, void *c, int m, int n, int k
     uint8_t *xws = (uint8_t *)workspace;
     uint8_t *wws = xws + operand_ws_bytes(m, k);
     hipError_t e = launch_convert_jobs(make_job(a, xws, m), make_job(b, wws, n), k, stream);
-    if (e == hipSuccess)
-        e = launch_fp6_gemm(xws, wws, c, m, n, k, ep, dev, stream);
-    return e;
+    if (e != hipSuccess)
+        return e;
+    // Few tiles and long K: K-slices of every tile on their own CUs, partial sums in slabs
+    // behind the operands, a second kernel for the sum and the epilogue.
+    const int ks = fp6_ksplit(m, n, k, dev);
+    if (ks == 1)
+        return launch_gemm_items(xws, wws, c, m, n, k, 1, ep, dev, stream);
+    int32_t *slabs = (int32_t *)(wws + operand_ws_bytes(n, k));
+    e = launch_gemm_items(xws, wws, slabs, m, n, k, ks, Epilogue{}, dev, stream);
+    if (e != hipSuccess)
+        return e;
+    const size_t count = (size_t)m * (size_t)n;
+    if (n % 4 == 0)
+        fp6_splitk_reduce_kernel<true><<<(unsigned)((count / 4 + 255) / 256), 256, 0, stream>>>(slabs, (int32_t *)c, count, ks, n, ep);
+    else
+        fp6_splitk_reduce_kernel<false><<<(unsigned)((count + 255) / 256), 256, 0, stream>>>(slabs, (int32_t *)c, count, ks, n, ep);
+    return hipGetLastError();
 }
 
 }  // namespace int4linear

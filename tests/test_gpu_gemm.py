@@ -247,6 +247,40 @@ def test_internal_workspace_shared_between_streams(gpu, host_threads):
         assert np.array_equal(yd.cpu().numpy(), want), f"case {i}"
 
 
+@pytest.mark.parametrize("m, n, k", [(300, 2049, 8192), (257, 1000, 4096), (512, 1024, 14336), (300, 520, 16392),
+                                     (1024, 4096, 14336)])
+def test_split_k_form_of_the_fp6_kernel(gpu, host_threads, m, n, k):
+    """64 tiles of 256 x 256 or fewer and long K: the FP6 GEMM runs K-slices of every tile on
+    their own CUs (partial sums in slabs behind the converted operands in the internal
+    workspace), a second kernel adds them up and applies the epilogue."""
+    import torch
+
+    import int4linear_amd as lib
+
+    x = helpers.uniform_s4(3200 + m, m, k)
+    w = helpers.uniform_s4(3300 + n, n, k)
+    want = oracle.linear_ref(x, w, threads=host_threads)
+    xp, wp = helpers.pack_bytes(x), helpers.pack_bytes(w)
+    lib.init()
+    operands = lib.fp6_operand_bytes(m, k) + lib.fp6_operand_bytes(n, k)
+    if lib.kernel_for_shape(m, n, k) == "fp6":
+        slabs = lib.workspace_bytes(m, n, k) - operands
+        assert slabs >= 2 * m * n * 4 and slabs % (m * n * 4) == 0
+    assert np.array_equal(helpers.run_gemm(xp, wp, m, n, k, kernel="fp6"), want)
+    rng = np.random.default_rng(m + k)
+    bias = rng.integers(-1000, 1000, size=n, dtype=np.int32)
+    rs = rng.uniform(0.1, 2.0, size=m).astype(np.float32)
+    cs = rng.uniform(0.1, 2.0, size=n).astype(np.float32)
+    xd, wd = helpers.to_device_bytes(xp), helpers.to_device_bytes(wp)
+    bd, rd, cd = (torch.from_numpy(a).to("cuda:0") for a in (bias, rs, cs))
+    y = torch.full((m, n), -1, dtype=torch.int32, device="cuda:0")
+    lib.linear_s32(xd, wd, bd, y, m, n, k, kernel="fp6")
+    assert np.array_equal(y.cpu().numpy(), oracle.epilogue(want, bias))
+    yf = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda:0")
+    lib.linear_f32(xd, wd, bd, rd, cd, yf, m, n, k, kernel="fp6")
+    assert np.array_equal(yf.cpu().numpy().view(np.int32), oracle.epilogue(want, bias, rs, cs, f32=True).view(np.int32))
+
+
 @pytest.mark.parametrize("m, n, k", [(128, 4096, 14336), (160, 4096, 4096), (300, 520, 4096), (1024, 512, 8192),
                                      (140, 1000, 4096), (200, 136, 16384)])
 def test_split_k_form_of_the_int8_kernel(gpu, host_threads, m, n, k):
