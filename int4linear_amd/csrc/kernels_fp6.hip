@@ -10,7 +10,7 @@
 // K * 64 < 2^24.  The launcher refuses larger K; the result is bit-identical to integer
 // arithmetic (the tests compare it against the CPU oracle).
 //
-// Two kernels:
+// Three kernels:
 //   * fp6_convert_kernel rewrites packed s4 operands (rows x K/2 bytes) into FP6
 //     "fragment-major" form in a workspace: for every block of 32 rows x 64 k the 24
 //     bytes each of the 64 MFMA lanes feeds to the instruction, stored as 64 x 16 B
@@ -21,7 +21,9 @@
 //     the workspace is already in the order lanes consume it, global->LDS is a linear
 //     direct-to-LDS copy, LDS->VGPR is one 16-byte and one 8-byte read per lane per
 //     fragment at consecutive addresses (no swizzle, no bank conflicts), and the main loop
-//     contains no VALU work at all.
+//     contains no VALU work at all.  With few output tiles and long K its work items are
+//     K-slices of tiles, which store partial sums into slabs of the workspace.
+//   * fp6_splitk_reduce_kernel adds those slabs up and applies the epilogue.
 //
 // Order of k inside a fragment is whatever the converter produces; it only has to be the
 // same for both operands, which it is because both go through the same converter.
