@@ -5,10 +5,13 @@
 // instruction does 32x32x32), and E2M3 holds every signed 4-bit integer exactly:
 // sign, two exponent bits and three mantissa bits encode n/8 for n = -15..15 as the plain
 // sign-magnitude integer |n| with the sign in bit 5 (subnormals 0..7 are |n| itself, 8 is
-// exponent 1 with mantissa 0).  With both block scales set to 2^3 a product is n*m
-// exactly, the fp32 accumulator holds integers, and fp32 is exact below 2^24, i.e. for
-// K * 64 < 2^24.  The launcher refuses larger K; the result is bit-identical to integer
-// arithmetic (the tests compare it against the CPU oracle).
+// exponent 1 with mantissa 0).  The instruction is used without block scales (both scale
+// arguments zero select the unscaled opcode, one instruction where the scaled one is a
+// pair), so a product is n*m/64, the fp32 accumulator holds multiples of 1/64, which fp32
+// represents exactly while |sum of n*m| < 2^24, i.e. for K * 64 < 2^24, and the store
+// multiplies by 64 (exact) before the conversion to int32.  The launcher refuses larger K;
+// the result is bit-identical to integer arithmetic (the tests compare it against the CPU
+// oracle).
 //
 // Three kernels:
 //   * fp6_convert_kernel rewrites packed s4 operands (rows x K/2 bytes) into FP6
@@ -62,7 +65,7 @@ constexpr int kLdsBytes = kStages * kStageBytes;                       // 144 Ki
 constexpr int kStaggerGroups = 8;                     // start groups within an XCD (power of two)
 constexpr int kStaggerTicks = 120;                    // delay between groups, in 10-ns ticks of the constant clock
 constexpr int kStaggerMinRounds = 2;                  // tiles per workgroup from which the start is staggered
-constexpr int kScale = 127 + 3;                       // E8M0 block scale 2^3 for both operands
+constexpr float kUnscale = 64.f;                      // the codes are n/8: a product is n*m/64
 
 // ---- converter --------------------------------------------------------------------------
 
@@ -380,8 +383,8 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
             ([&] {
                 constexpr int j = SLOT / C::FN, i = SLOT % C::FN;
                 acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                    frag(xlo[p][j], xhi[p][j]), frag(wlo[p][i], whi[p][i]), acc[i][j], 2, 2, 0, kScale, 0,
-                    kScale);
+                    frag(xlo[p][j], xhi[p][j]), frag(wlo[p][i], whi[p][i]), acc[i][j], 2, 2, 0, 0, 0,
+                    0);
                 // An MFMA has no side effect, so nothing stops the optimiser from moving it
                 // down to its next use, past the housekeeping meant to run in its shadow;
                 // this empty statement "uses" the result here and keeps the MFMA in place.
@@ -515,7 +518,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
                         const unsigned row_off = lm + dm < rows_left ? lm_off + (unsigned)dm * (unsigned)N * 4u : 0x80000000u;
 #pragma unroll
                         for (int i = 0; i < C::FN; ++i) {
-                            const int v = (int)acc[i][j][t];
+                            const int v = (int)(acc[i][j][t] * kUnscale);
                             __builtin_amdgcn_raw_buffer_store_b32((unsigned)v, rsrc, row_off + col_off[i], 0, 2 /* nt */);
                         }
                     }
@@ -548,7 +551,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
                         const unsigned row_off = lm + dm < rows_left ? lm_off + (unsigned)dm * (unsigned)N * 4u : 0x80000000u;
 #pragma unroll
                         for (int i = 0; i < C::FN; ++i) {
-                            const int v = epilogue_value(ep, (int)acc[i][j][t], bias_v[i], rs[t], cs_v[i]);
+                            const int v = epilogue_value(ep, (int)(acc[i][j][t] * kUnscale), bias_v[i], rs[t], cs_v[i]);
                             __builtin_amdgcn_raw_buffer_store_b32((unsigned)v, rsrc, row_off + col_off[i], 0, 2 /* nt */);
                         }
                     }
