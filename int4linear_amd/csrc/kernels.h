@@ -92,4 +92,9 @@ hipError_t launch_unpack(const int *src, int *dst, int m, int n, hipStream_t str
 // Fill `count` int32 words with zero (a kernel, so callers may capture it in a graph).
 hipError_t launch_zero_i32(int *dst, size_t count, hipStream_t stream);
 
+// Second kernel of the split-K forms: c = epilogue(sum of the ksplit slabs of count = m * n
+// partial sums each that lie back to back at `slabs`, 16-byte aligned).
+hipError_t launch_splitk_reduce(const void *slabs, void *c, size_t count, int ksplit, int n, const Epilogue &ep,
+                                hipStream_t stream);
+
 }  // namespace int4linear

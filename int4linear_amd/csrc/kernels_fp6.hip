@@ -13,7 +13,7 @@
 // the result is bit-identical to integer arithmetic (the tests compare it against the CPU
 // oracle).
 //
-// Three kernels:
+// Two kernels:
 //   * fp6_convert_kernel rewrites packed s4 operands (rows x K/2 bytes) into FP6
 //     "fragment-major" form in a workspace: for every block of 32 rows x 64 k the 24
 //     bytes each of the 64 MFMA lanes feeds to the instruction, stored as 64 x 16 B
@@ -26,7 +26,7 @@
 //     fragment at consecutive addresses (no swizzle, no bank conflicts), and the main loop
 //     contains no VALU work at all.  With few output tiles and long K its work items are
 //     K-slices of tiles, which store partial sums into slabs of the workspace.
-//   * fp6_splitk_reduce_kernel adds those slabs up and applies the epilogue.
+//     (launch_splitk_reduce adds those slabs up and applies the epilogue).
 //
 // Order of k inside a fragment is whatever the converter produces; it only has to be the
 // same for both operands, which it is because both go through the same converter.
@@ -678,41 +678,6 @@ hipError_t launch_gemm_items(const void *a_conv, const void *b_conv, void *c, in
     return hipGetLastError();
 }
 
-// Second kernel of the split-K form: Y = epilogue(sum of the ksplit slabs), four outputs of
-// one row per thread (VEC: n % 4 == 0) or one.
-template <bool VEC>
-__global__ __launch_bounds__(256) void fp6_splitk_reduce_kernel(const int32_t *__restrict__ partial,
-                                                                int32_t *__restrict__ Y, size_t count, int ksplit,
-                                                                int N, Epilogue ep)
-{
-    constexpr int kPer = VEC ? 4 : 1;
-    const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * kPer;
-    if (i >= count)
-        return;
-    int sum[kPer] = {};
-    for (int s = 0; s < ksplit; ++s) {
-        const int32_t *src = partial + (size_t)s * count + i;
-        if constexpr (VEC) {
-            const v4i v = __builtin_nontemporal_load((const v4i *)src);
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-                sum[q] += v[q];
-        } else {
-            sum[0] += *src;
-        }
-    }
-    const size_t row = i / (size_t)N;
-    const int col = (int)(i - row * (size_t)N);
-    const float rs = ep.row_scale ? ep.row_scale[row] : 1.f;
-#pragma unroll
-    for (int q = 0; q < kPer; ++q)
-        sum[q] = epilogue_value(ep, sum[q], ep.bias ? ep.bias[col + q] : 0, rs, ep.col_scale ? ep.col_scale[col + q] : 1.f);
-    if constexpr (VEC)
-        *(v4i *)(Y + i) = (v4i){sum[0], sum[1], sum[2], sum[3]};
-    else
-        Y[i] = sum[0];
-}
-
 }  // namespace
 
 hipError_t launch_fp6_gemm(const void *a_conv, const void *b_conv, void *c, int m, int n, int k,
@@ -738,12 +703,7 @@ hipError_t launch_fp6(const void *a, const void *b, void *c, int m, int n, int k
     e = launch_gemm_items(xws, wws, slabs, m, n, k, ks, Epilogue{}, dev, stream);
     if (e != hipSuccess)
         return e;
-    const size_t count = (size_t)m * (size_t)n;
-    if (n % 4 == 0)
-        fp6_splitk_reduce_kernel<true><<<(unsigned)((count / 4 + 255) / 256), 256, 0, stream>>>(slabs, (int32_t *)c, count, ks, n, ep);
-    else
-        fp6_splitk_reduce_kernel<false><<<(unsigned)((count + 255) / 256), 256, 0, stream>>>(slabs, (int32_t *)c, count, ks, n, ep);
-    return hipGetLastError();
+    return launch_splitk_reduce(slabs, c, (size_t)m * (size_t)n, ks, n, ep, stream);
 }
 
 }  // namespace int4linear

@@ -570,23 +570,6 @@ using CfgLarge = TileConfig<2, 4, 4, 2, 4, 1>;
 // whose 256 x 256 tile count would leave CUs idle.
 using CfgMedium = TileConfig<2, 2, 2, 2, 4, 2>;
 
-// Second kernel of the split-K path: Y[i][j] = epilogue(sum over the ksplit partial slabs).
-__global__ __launch_bounds__(256) void splitk_reduce_kernel(const int32_t *__restrict__ partial,
-                                                            int32_t *__restrict__ Y, size_t count, int ksplit,
-                                                            int N, Epilogue ep)
-{
-    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= count)
-        return;
-    int sum = 0;
-    for (int s = 0; s < ksplit; ++s)
-        sum += partial[(size_t)s * count + i];
-    const size_t row = i / (size_t)N;
-    const int col = (int)(i - row * (size_t)N);
-    Y[i] = epilogue_value(ep, sum, ep.bias ? ep.bias[col] : 0, ep.row_scale ? ep.row_scale[row] : 1.f,
-                          ep.col_scale ? ep.col_scale[col] : 1.f);
-}
-
 template <class C>
 hipError_t set_lds_limit()
 {
@@ -684,10 +667,7 @@ hipError_t launch_mfma_splitk(const void *a, const void *b, void *c, int m, int 
     hipError_t e = launch_cfg<CfgMedium>(a, b, workspace, m, n, k, Epilogue{}, dev, stream, d);
     if (e != hipSuccess)
         return e;
-    const size_t count = (size_t)m * (size_t)n;
-    splitk_reduce_kernel<<<(unsigned)((count + 255) / 256), 256, 0, stream>>>((const int32_t *)workspace, (int32_t *)c,
-                                                                              count, d, n, ep);
-    return hipGetLastError();
+    return launch_splitk_reduce(workspace, c, (size_t)m * (size_t)n, d, n, ep, stream);
 }
 
 hipError_t launch_mfma(const void *a, const void *b, void *c, int m, int n, int k,

@@ -95,6 +95,43 @@ __global__ void zero_i32_kernel(int4 *__restrict__ dst4, int *__restrict__ dst, 
         dst[t] = 0;
 }
 
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+// Second kernel of the split-K forms: Y = epilogue(sum of the ksplit slabs), four outputs of
+// one row per thread (VEC: n % 4 == 0) or one.
+template <bool VEC>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const int32_t *__restrict__ partial,
+                                                                int32_t *__restrict__ Y, size_t count, int ksplit,
+                                                                int N, Epilogue ep)
+{
+    constexpr int kPer = VEC ? 4 : 1;
+    const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * kPer;
+    if (i >= count)
+        return;
+    int sum[kPer] = {};
+    for (int s = 0; s < ksplit; ++s) {
+        const int32_t *src = partial + (size_t)s * count + i;
+        if constexpr (VEC) {
+            const v4i v = __builtin_nontemporal_load((const v4i *)src);
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                sum[q] += v[q];
+        } else {
+            sum[0] += *src;
+        }
+    }
+    const size_t row = i / (size_t)N;
+    const int col = (int)(i - row * (size_t)N);
+    const float rs = ep.row_scale ? ep.row_scale[row] : 1.f;
+#pragma unroll
+    for (int q = 0; q < kPer; ++q)
+        sum[q] = epilogue_value(ep, sum[q], ep.bias ? ep.bias[col + q] : 0, rs, ep.col_scale ? ep.col_scale[col + q] : 1.f);
+    if constexpr (VEC)
+        *(v4i *)(Y + i) = (v4i){sum[0], sum[1], sum[2], sum[3]};
+    else
+        Y[i] = sum[0];
+}
+
 }  // namespace
 
 hipError_t launch_simple(const void *a, const void *b, void *c, int m, int n, int k,
@@ -142,6 +179,20 @@ hipError_t launch_zero_i32(int *dst, size_t count, hipStream_t stream)
     size_t want = (vec_count + block - 1) / block;
     unsigned grid = (unsigned)(want < 1 ? 1 : (want > 8192 ? 8192 : want));
     zero_i32_kernel<<<grid, block, 0, stream>>>((int4 *)dst, dst, vec_count, count);
+    return hipGetLastError();
+}
+
+hipError_t launch_splitk_reduce(const void *slabs, void *c, size_t count, int ksplit, int n, const Epilogue &ep,
+                                hipStream_t stream)
+{
+    if (count == 0)
+        return hipSuccess;
+    if (n % 4 == 0)
+        splitk_reduce_kernel<true><<<(unsigned)((count / 4 + 255) / 256), 256, 0, stream>>>(
+            (const int32_t *)slabs, (int32_t *)c, count, ksplit, n, ep);
+    else
+        splitk_reduce_kernel<false><<<(unsigned)((count + 255) / 256), 256, 0, stream>>>(
+            (const int32_t *)slabs, (int32_t *)c, count, ksplit, n, ep);
     return hipGetLastError();
 }
 
