@@ -269,19 +269,6 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
     if (bid >= total_tiles)
         return;
     const int my_tiles = (total_tiles - bid + nblk - 1) / nblk;
-    // Workgroups that start together reach every tile end together, and the stores of all
-    // tiles then queue for the same path to memory while no CU computes.  With two or
-    // more tiles per workgroup the 32 workgroups of an XCD (ids congruent mod 8) therefore
-    // start in eight groups about a microsecond apart: their tile ends stay that
-    // far apart for the rest of the launch, which costs the spread once at the end and
-    // saves most of the wait at every tile end before.
-    if (total_tiles >= kStaggerMinRounds * nblk) {
-        const int grp = (bid >> 3) & (kStaggerGroups - 1);
-        const unsigned long long until = wall_clock64() + (unsigned long long)(grp * kStaggerTicks);
-        while (wall_clock64() < until)
-            __builtin_amdgcn_s_sleep(2);
-    }
-
     // ---- load side: stage = 24 KiB of X fragments then 24 KiB of W fragments, copied
     //      linearly; wave w moves CH/2 consecutive 1-KiB chunks of either half, so that the
     //      chunks of a half differ only in the instruction's constant.
@@ -412,6 +399,20 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
             ld_chunk(std::integral_constant<int, decltype(half_pos)::value * (C::CH / 2) + slot - kDmaFirstSlot>{}, load_ring);
         }
     };
+
+    // Workgroups that start together reach every tile end together, and the stores of all
+    // tiles then queue for the same path to memory while no CU computes.  With two or
+    // more tiles per workgroup the 32 workgroups of an XCD (ids congruent mod 8) therefore
+    // start in eight groups about a microsecond apart: their tile ends stay that
+    // far apart for the rest of the launch, which costs the spread once at the end and
+    // saves most of the wait at every tile end before.  (The wait sits behind the first loads,
+    // which travel meanwhile.)
+    if (total_tiles >= kStaggerMinRounds * nblk) {
+        const int grp = (bid >> 3) & (kStaggerGroups - 1);
+        const unsigned long long until = wall_clock64() + (unsigned long long)(grp * kStaggerTicks);
+        while (wall_clock64() < until)
+            __builtin_amdgcn_s_sleep(2);
+    }
 
     // Stage 0 must have landed before the first read; stage 1 and half of stage 2 are
     // in flight behind it.
