@@ -88,14 +88,14 @@ bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 // bytes of HBM traffic).  Measured against the int8 kernel (tiles, K -> faster kernel):
 // 128, 4096 -> tie; 128, 8192 -> FP6 by 8 %; 128, 14336 -> FP6 by 20 %; 144, 3072 -> FP6;
 // 256, 2048 -> int8 by 5 %; 512, 2048 -> FP6 by 20 %; 512, 1024 -> FP6 by 3 %; 1024, 1024
-// -> tie; 1024, 512 -> int8 by 10 %.  Split over K (64 tiles or fewer on 256 CUs): 64 tiles
-// at K = 14336 -> FP6 by 9 %, at K = 28672 by 16 %; 48 tiles at K = 8192 and 32 or fewer
-// at K = 14336 -> int8 (itself split over K).
+// -> tie; 1024, 512 -> int8 by 10 %.  With 64 tiles or fewer the FP6 GEMM splits K, but the
+// int8 kernel's small-grid form is as fast or faster there (64 tiles: 62 against 81 us at
+// K = 14336, 122 against 131 and 115 against 109 us at K = 28672), so the automatic choice
+// leaves those shapes to it.
 bool fp6_worthwhile(int m, int n, int k, const DeviceInfo &dev)
 {
     const long tiles = (long)((m + 255) / 256) * ((n + 255) / 256);
-    const bool pays = (tiles >= 128 && k >= 8192) || (tiles >= 144 && k >= 3072) || (tiles >= 384 && k >= 1024) ||
-                      (tiles >= 64 && k >= 12288 && fp6_ksplit(m, n, k, dev) > 1);
+    const bool pays = (tiles >= 128 && k >= 8192) || (tiles >= 144 && k >= 3072) || (tiles >= 384 && k >= 1024);
     return pays && fp6_supports(m, n, k) && fp6_workspace_bytes(m, n, k, dev) <= g_workspace_limit.load();
 }
 

@@ -563,6 +563,199 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
     __builtin_amdgcn_s_waitcnt(I4L_VMCNT(0));
 }
 
+// ---- the form for grids of a few tiles per CU -----------------------------------------
+//
+// With one 128 x 128 tile per CU the kernel above has a single wave per SIMD (two with two
+// tiles), and a single wave cannot issue the nibble widening and the MFMAs fast enough to
+// keep the matrix pipe busy (about 90 cycles per 32-cycle MFMA).  Here the tile has eight waves: wave w owns the
+// 64 x 64 quadrant w % 4 of C together with wave w ^ 4, and the two (they share a SIMD)
+// split every stage's K between them: group w / 4 takes half w / 4 of the stage's 128 k (the
+// 16-byte chunks 2h and 2h + 1 of a row).  Each wave thus widens the same four fragments per
+// eight MFMAs as before but has half of everything to issue, and the pipe is fed by two
+// instruction streams.  At the tile's end the upper group hands its accumulators to the
+// lower one through LDS.  One tile per workgroup, a four-stage ring of 16 KiB stages, two
+// direct-to-LDS loads per wave and stage, one barrier per stage.
+constexpr int kPairTile = 128;
+constexpr int kPairStages = 4;
+constexpr int kPairStageBytes = 2 * kPairTile * kRowBytes;    // 16 KiB: X rows, then W rows
+constexpr int kPairLdsBytes = kPairStages * kPairStageBytes;  // 64 KiB, also the merge area
+constexpr int kPairRounds = 2;  // used up to this many tiles per CU (two workgroups fit a CU); measured: beyond, the 256 x 256 tiles win
+
+__global__ __launch_bounds__(512) void mfma_pair_kernel(const uint8_t *__restrict__ X,
+                                                        const uint8_t *__restrict__ W,
+                                                        int32_t *__restrict__ Y, int M, int N, int K,
+                                                        int tiles_m, int tiles_n, Epilogue ep)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int half = wave >> 2;  // which half of every stage's K
+    const int quad = wave & 3;
+    const int wm = quad >> 1, wn = quad & 1;
+    const int rowbytes = K >> 1;
+    const int KT = K / kStageK;
+    int tm, tn;
+    tile_coords(blockIdx.x, tiles_m * tiles_n, tiles_m, tiles_n, tm, tn);
+    const int m0 = tm * kPairTile, n0 = tn * kPairTile;
+
+    // ---- loads: wave w moves the 16-row chunk w of the X rows and of the W rows of every
+    //      stage.  Lane p lands at byte 16 p of the chunk: row p / 4, slot p % 4, and fetches
+    //      the row's chunk slot ^ swz(row).  Rows past the matrix re-read its last row.
+    const int ld_row = lane >> 2;
+    const int ld_c = (lane & 3) ^ swz(ld_row);
+    const int xr = min(wave * kChunkRows + ld_row, M - 1 - m0);
+    const int wr = min(wave * kChunkRows + ld_row, N - 1 - n0);
+    const unsigned voff_x = (unsigned)xr * (unsigned)rowbytes + (unsigned)ld_c * 16u;
+    const unsigned voff_w = (unsigned)wr * (unsigned)rowbytes + (unsigned)ld_c * 16u;
+    const uint8_t *xptr = X + (size_t)m0 * rowbytes;
+    const uint8_t *wptr = W + (size_t)n0 * rowbytes;
+    const unsigned lds_base = (unsigned)(size_t)I4L_LDS(lds);
+    const unsigned place_x = lds_base + (unsigned)(wave * kChunkBytes);
+    const unsigned place_w = place_x + (unsigned)(kPairTile * kRowBytes);
+    // Stage st into ring position st % 4.  Past the last stage the last one is fetched
+    // again, into a buffer nobody reads any more, so that every iteration issues the same
+    // number of loads and the wait below is a constant.
+    auto issue = [&](int st) {
+        const int src = st < KT ? st : KT - 1;
+        const unsigned ring = (unsigned)((st % kPairStages) * kPairStageBytes);
+        dma16(xptr + (size_t)src * kRowBytes, voff_x, place_x, ring);
+        dma16(wptr + (size_t)src * kRowBytes, voff_w, place_w, ring);
+    };
+#pragma unroll
+    for (int st = 0; st < kPairStages - 1; ++st)
+        issue(st);
+
+    // ---- math: lane (fr, fg) supplies row fr of a 32-row fragment and, of this wave's half
+    //      of the stage, the 16-byte chunk fg (32 nibbles: the even ones feed one MFMA, the
+    //      odd ones the next).
+    const int fr = lane & 31;
+    const int fg = lane >> 5;
+    const unsigned rd_off = (unsigned)fr * kRowBytes + (unsigned)(((2 * half + fg) ^ swz(fr)) * 16);
+    const unsigned x_rd = (unsigned)(wm * 64 * kRowBytes) + rd_off;
+    const unsigned w_rd = (unsigned)((kPairTile + wn * 64) * kRowBytes) + rd_off;
+    const int himask = (int)0xF0F0F0F0u;
+    v16i acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int t = 0; t < 16; ++t)
+                acc[i][j][t] = 0;
+
+    // The MFMAs of a stage are issued one iteration late, behind the LDS reads of the next
+    // stage, so that those reads (and the widening that waits for them) run in their shadow.
+    v4i xlo[2], xhi[2], wlo[2], whi[2];
+    auto multiply = [&]() {
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(xlo[j], wlo[i], acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(xhi[j], whi[i], acc[i][j], 0, 0, 0);
+            }
+    };
+#pragma unroll 1
+    for (int st = 0; st < KT; ++st) {
+        // Stage st has landed once this wave's two loads of it have (the loads of the two
+        // younger stages may still be in flight) and every wave has said the same; by then
+        // every wave has also finished reading stage st - 1, whose buffer the loads of
+        // stage st + 3 now refill.
+        __builtin_amdgcn_s_waitcnt(I4L_VMCNT(2 * (kPairStages - 2)));
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        issue(st + kPairStages - 1);
+        const uint8_t *stage = lds + (st % kPairStages) * kPairStageBytes;
+        v4i px[2], pw[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+            px[j] = *(const v4i *)(stage + x_rd + j * kFrag * kRowBytes);
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+            pw[i] = *(const v4i *)(stage + w_rd + i * kFrag * kRowBytes);
+        if (st > 0)
+            multiply();  // stage st - 1
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            xlo[j] = (px[j] << 4) & himask;
+            xhi[j] = px[j] & himask;
+            wlo[j] = (pw[j] << 4) & himask;
+            whi[j] = pw[j] & himask;
+        }
+    }
+    multiply();  // the last stage
+
+    // ---- the upper group's sums go through LDS to the lower group, which stores the tile.
+    //      Register r of lane l of quadrant q sits at word (q * 64 + r) * 64 + l.
+    __builtin_amdgcn_s_waitcnt(I4L_VMCNT(0));  // the loads past the end have landed too
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    int *merge = (int *)lds + (size_t)quad * 64 * 64 + lane;
+    if (half == 1) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int t = 0; t < 16; ++t)
+                    merge[((i * 2 + j) * 16 + t) * 64] = acc[i][j][t];
+    }
+    __syncthreads();
+    if (half == 1)
+        return;
+    // X is the MFMA A operand: accumulator t of fragment (i, j) is
+    //   m = 32 j + 8 (t / 4) + 4 (lane / 32) + t % 4,  n = 32 i + lane % 32.
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int t = 0; t < 16; ++t)
+                acc[i][j][t] = (acc[i][j][t] + merge[((i * 2 + j) * 16 + t) * 64]) >> 8;  // both operands carried a factor 16
+    const int mw = m0 + wm * 64 + 4 * (lane >> 5);
+    const int nw = n0 + wn * 64 + (lane & 31);
+    int32_t *out = Y + (size_t)mw * N + nw;
+    if (!ep.bias && !ep.row_scale && !ep.col_scale && !ep.f32) {
+        // nothing to load: the stores follow one another without a wait
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int t = 0; t < 16; ++t) {
+                const int dm = 32 * j + 8 * (t / 4) + (t % 4);
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+                    if (mw + dm < M && nw + 32 * i < N)
+                        out[(size_t)dm * N + 32 * i] = acc[i][j][t];
+            }
+        return;
+    }
+    // The epilogue's operands of this lane's columns and rows (clamped inside the matrix)
+    // are fetched before the first store, so that no store waits for a load behind it.
+    int bias_v[2];
+    float cs_v[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int nn = min(nw + 32 * i, N - 1);
+        bias_v[i] = ep.bias ? ep.bias[nn] : 0;
+        cs_v[i] = ep.col_scale ? ep.col_scale[nn] : 1.f;
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        float rs[16];
+#pragma unroll
+        for (int t = 0; t < 16; ++t)
+            rs[t] = ep.row_scale ? ep.row_scale[min(mw + 32 * j + 8 * (t / 4) + (t % 4), M - 1)] : 1.f;
+#pragma unroll
+        for (int t = 0; t < 16; ++t) {
+            const int dm = 32 * j + 8 * (t / 4) + (t % 4);
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+                if (mw + dm < M && nw + 32 * i < N)
+                    out[(size_t)dm * N + 32 * i] = epilogue_value(ep, acc[i][j][t], bias_v[i], rs[t], cs_v[i]);
+        }
+    }
+}
+
 // 256 x 256 tile, eight wavefronts of 128 (m) x 64 (n), one workgroup per CU, two
 // wavefronts per SIMD: the large-shape configuration.
 using CfgLarge = TileConfig<2, 4, 4, 2, 4, 1>;
@@ -627,8 +820,9 @@ hipError_t launch_mfma_tile(const void *a, const void *b, void *c, int m, int n,
 }
 
 // K-slices per tile for shapes whose 128 x 128 tiles would fill at most an eighth of the
-// device at K >= 4096, or at most half of it at K >= 8192 (measured: with more tiles or
-// shorter K the second pass over the partial sums costs more than the idle CUs): the largest divisor of the stage count
+// device's 512 slots at K >= 4096, or less than a quarter of them at K >= 8192 (measured
+// against the unsplit small-grid form: with more tiles or shorter K the second pass over the
+// partial sums costs more than the idle CUs): the largest divisor of the stage count
 // that keeps at least eight stages per slice, at most eight slices, and at most half a
 // work item per slot.
 int mfma_ksplit(int m, int n, int k, const DeviceInfo &dev)
@@ -639,7 +833,7 @@ int mfma_ksplit(int m, int n, int k, const DeviceInfo &dev)
     const long slots = (long)dev.cu_count * CfgMedium::OCC;
     const int stages = k / kStageK;
     const bool few_tiles = tiles * 8 <= slots && stages >= 32;
-    const bool long_k = tiles * 2 <= slots && stages >= 64;
+    const bool long_k = tiles * 4 < slots && stages >= 64;
     if (!few_tiles && !long_k)
         return 1;
     long limit = slots / (2 * tiles);
@@ -675,6 +869,13 @@ hipError_t launch_mfma(const void *a, const void *b, void *c, int m, int n, int 
 {
     const long tiles_large = (long)((m + CfgLarge::BM - 1) / CfgLarge::BM) *
                              ((n + CfgLarge::BN - 1) / CfgLarge::BN);
+    // Few 128 x 128 tiles per CU: the form whose two waves per SIMD split K.
+    const int pair_m = (m + kPairTile - 1) / kPairTile, pair_n = (n + kPairTile - 1) / kPairTile;
+    if ((long)pair_m * pair_n <= (long)dev.cu_count * kPairRounds) {
+        mfma_pair_kernel<<<(unsigned)(pair_m * pair_n), 512, kPairLdsBytes, stream>>>(
+            (const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k, pair_m, pair_n, ep);
+        return hipGetLastError();
+    }
     // Use the big tile once it alone can occupy every CU.
     if (tiles_large >= dev.cu_count)
         return launch_cfg<CfgLarge>(a, b, c, m, n, k, ep, dev, stream);

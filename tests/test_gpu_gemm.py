@@ -247,6 +247,37 @@ def test_internal_workspace_shared_between_streams(gpu, host_threads):
         assert np.array_equal(yd.cpu().numpy(), want), f"case {i}"
 
 
+@pytest.mark.parametrize("m, n, k", [(128, 128, 128), (1, 1, 128), (129, 257, 384), (1000, 3000, 1024), (2048, 2048, 256),
+                                     (777, 1531, 2048), (2048, 4096, 512)])
+def test_small_grid_form_of_the_int8_kernel(gpu, host_threads, m, n, k):
+    """Up to two 128 x 128 tiles per CU the int8 kernel runs in the form whose two waves per
+    SIMD split every stage's K and merge their sums through LDS: plain and with every
+    epilogue, ragged edges in both directions, one to many stages."""
+    import torch
+
+    import int4linear_amd as lib
+
+    x = helpers.uniform_s4(4200 + m, m, k)
+    w = helpers.uniform_s4(4300 + n, n, k)
+    want = oracle.linear_ref(x, w, threads=host_threads)
+    xp, wp = helpers.pack_bytes(x), helpers.pack_bytes(w)
+    assert np.array_equal(helpers.run_gemm(xp, wp, m, n, k, kernel="mfma"), want)
+    rng = np.random.default_rng(m + n + k)
+    bias = rng.integers(-1000, 1000, size=n, dtype=np.int32)
+    rs = rng.uniform(0.1, 2.0, size=m).astype(np.float32)
+    cs = rng.uniform(0.1, 2.0, size=n).astype(np.float32)
+    xd, wd = helpers.to_device_bytes(xp), helpers.to_device_bytes(wp)
+    bd, rd, cd = (torch.from_numpy(a).to("cuda:0") for a in (bias, rs, cs))
+    y = torch.full((m, n), -1, dtype=torch.int32, device="cuda:0")
+    lib.linear_s32(xd, wd, bd, y, m, n, k, kernel="mfma")
+    assert np.array_equal(y.cpu().numpy(), oracle.epilogue(want, bias))
+    yf = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda:0")
+    lib.linear_f32(xd, wd, bd, rd, cd, yf, m, n, k, kernel="mfma")
+    assert np.array_equal(yf.cpu().numpy().view(np.int32), oracle.epilogue(want, bias, rs, cs, f32=True).view(np.int32))
+    lib.linear_f32(xd, wd, None, rd, None, yf, m, n, k, kernel="mfma")
+    assert np.array_equal(yf.cpu().numpy().view(np.int32), oracle.epilogue(want, None, rs, None, f32=True).view(np.int32))
+
+
 @pytest.mark.parametrize("m, n, k", [(300, 2049, 8192), (257, 1000, 4096), (512, 1024, 14336), (300, 520, 16392),
                                      (1024, 4096, 14336)])
 def test_split_k_form_of_the_fp6_kernel(gpu, host_threads, m, n, k):
