@@ -335,7 +335,7 @@ def main() -> int:
     tops_wall = ops / (wall_ms * 1e-3) / 1e12
     # The roofline that bounds the dominant kernel is that of the MFMA type it issues.
     peak = FP6_MFMA_PEAK_TOPS if kernel == "fp6" else INT8_MFMA_PEAK_TOPS
-    kernel_name = {"fp6": "fp6_gemm_kernel (v_mfma_scale_f32_32x32x64_f8f6f4, E2M3 operands)",
+    kernel_name = {"fp6": "fp6_gemm_kernel (v_mfma_f32_32x32x64_f8f6f4, E2M3 operands)",
                    "mfma": "mfma_gemm_kernel (v_mfma_i32_32x32x32_i8)"}.get(kernel, kernel)
 
     result = {

@@ -45,13 +45,14 @@ enum {
 enum {
     INT4LINEAR_KERNEL_AUTO = 0,   /* shape-based dispatch (what the plain entry uses)    */
     INT4LINEAR_KERNEL_SIMPLE = 1, /* one thread per output, scalar nibble decode; any K%8==0 */
-    INT4LINEAR_KERNEL_MFMA = 2,   /* LDS-pipelined v_mfma_i32_32x32x32_i8 kernel; K%128==0 */
+    INT4LINEAR_KERNEL_MFMA = 2,   /* LDS-pipelined v_mfma_i32_32x32x32_i8 kernel (tile and form
+                                     chosen from the grid); K%128==0 */
     INT4LINEAR_KERNEL_SKINNY = 3, /* weight-streaming kernel: M <= 64 and K%128==0, or more
                                      rows (in runs of 64) when K splits into 128-byte tiles */
     INT4LINEAR_KERNEL_FP6 = 4,    /* operands converted to FP6 (E2M3) in a workspace, then
-                                     v_mfma_scale_f32_32x32x64_f8f6f4; exact; any K%8==0
+                                     v_mfma_f32_32x32x64_f8f6f4; exact; any K%8==0
                                      below 2^18 (the converter pads K to 128 with zeros) */
-    INT4LINEAR_KERNEL_MFMA_128 = 5, /* the int8 kernel with its 128x128 workgroup tile   */
+    INT4LINEAR_KERNEL_MFMA_128 = 5, /* the int8 kernel's pipelined form, 128x128 workgroup tile */
     INT4LINEAR_KERNEL_MFMA_256 = 6  /* the int8 kernel with its 256x256 workgroup tile   */
 };
 
