@@ -584,7 +584,7 @@ constexpr int kPairRounds = 2;  // used up to this many tiles per CU (two workgr
 __global__ __launch_bounds__(512) void mfma_pair_kernel(const uint8_t *__restrict__ X,
                                                         const uint8_t *__restrict__ W,
                                                         int32_t *__restrict__ Y, int M, int N, int K,
-                                                        int tiles_m, int tiles_n, Epilogue ep)
+                                                        int tiles_m, int tiles_n, int ksplit, Epilogue ep)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int lane = threadIdx.x & 63;
@@ -593,10 +593,15 @@ __global__ __launch_bounds__(512) void mfma_pair_kernel(const uint8_t *__restric
     const int quad = wave & 3;
     const int wm = quad >> 1, wn = quad & 1;
     const int rowbytes = K >> 1;
-    const int KT = K / kStageK;
+    // With ksplit > 1 workgroup v is K-slice v / tiles of tile v % tiles: it covers KT of the
+    // stages and stores plain partial sums into slab v / tiles of Y (M * N int32 each).
+    const int tiles = tiles_m * tiles_n;
+    const int slice = blockIdx.x / tiles;
+    const int KT = K / kStageK / ksplit;
     int tm, tn;
-    tile_coords(blockIdx.x, tiles_m * tiles_n, tiles_m, tiles_n, tm, tn);
+    tile_coords(blockIdx.x - slice * tiles, tiles, tiles_m, tiles_n, tm, tn);
     const int m0 = tm * kPairTile, n0 = tn * kPairTile;
+    Y += (size_t)slice * (size_t)M * (size_t)N;
 
     // ---- loads: wave w moves the 16-row chunk w of the X rows and of the W rows of every
     //      stage.  Lane p lands at byte 16 p of the chunk: row p / 4, slot p % 4, and fetches
@@ -607,8 +612,8 @@ __global__ __launch_bounds__(512) void mfma_pair_kernel(const uint8_t *__restric
     const int wr = min(wave * kChunkRows + ld_row, N - 1 - n0);
     const unsigned voff_x = (unsigned)xr * (unsigned)rowbytes + (unsigned)ld_c * 16u;
     const unsigned voff_w = (unsigned)wr * (unsigned)rowbytes + (unsigned)ld_c * 16u;
-    const uint8_t *xptr = X + (size_t)m0 * rowbytes;
-    const uint8_t *wptr = W + (size_t)n0 * rowbytes;
+    const uint8_t *xptr = X + (size_t)m0 * rowbytes + (size_t)slice * KT * kRowBytes;
+    const uint8_t *wptr = W + (size_t)n0 * rowbytes + (size_t)slice * KT * kRowBytes;
     const unsigned lds_base = (unsigned)(size_t)I4L_LDS(lds);
     const unsigned place_x = lds_base + (unsigned)(wave * kChunkBytes);
     const unsigned place_w = place_x + (unsigned)(kPairTile * kRowBytes);
@@ -711,11 +716,11 @@ __global__ __launch_bounds__(512) void mfma_pair_kernel(const uint8_t *__restric
         for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int t = 0; t < 16; ++t)
-                acc[i][j][t] = (acc[i][j][t] + merge[((i * 2 + j) * 16 + t) * 64]) >> 8;  // both operands carried a factor 16
+                acc[i][j][t] = (acc[i][j][t] + merge[((i * 2 + j) * 16 + t) * 64]) >> 8;  // both operands carried a factor 16 (exact per slice: every product is a multiple of 256)
     const int mw = m0 + wm * 64 + 4 * (lane >> 5);
     const int nw = n0 + wn * 64 + (lane & 31);
     int32_t *out = Y + (size_t)mw * N + nw;
-    if (!ep.bias && !ep.row_scale && !ep.col_scale && !ep.f32) {
+    if (ksplit > 1 || (!ep.bias && !ep.row_scale && !ep.col_scale && !ep.f32)) {
         // nothing to load: the stores follow one another without a wait
 #pragma unroll
         for (int j = 0; j < 2; ++j)
@@ -858,7 +863,11 @@ hipError_t launch_mfma_splitk(const void *a, const void *b, void *c, int m, int 
     const int d = mfma_ksplit(m, n, k, dev);
     if (d <= 1 || !workspace)
         return launch_mfma(a, b, c, m, n, k, ep, dev, stream);
-    hipError_t e = launch_cfg<CfgMedium>(a, b, workspace, m, n, k, Epilogue{}, dev, stream, d);
+    // the K-slices run as work items of the small-grid form
+    const int pair_m = (m + kPairTile - 1) / kPairTile, pair_n = (n + kPairTile - 1) / kPairTile;
+    mfma_pair_kernel<<<(unsigned)(pair_m * pair_n * d), 512, kPairLdsBytes, stream>>>(
+        (const uint8_t *)a, (const uint8_t *)b, (int32_t *)workspace, m, n, k, pair_m, pair_n, d, Epilogue{});
+    hipError_t e = hipGetLastError();
     if (e != hipSuccess)
         return e;
     return launch_splitk_reduce(workspace, c, (size_t)m * (size_t)n, d, n, ep, stream);
@@ -873,7 +882,7 @@ hipError_t launch_mfma(const void *a, const void *b, void *c, int m, int n, int 
     const int pair_m = (m + kPairTile - 1) / kPairTile, pair_n = (n + kPairTile - 1) / kPairTile;
     if ((long)pair_m * pair_n <= (long)dev.cu_count * kPairRounds) {
         mfma_pair_kernel<<<(unsigned)(pair_m * pair_n), 512, kPairLdsBytes, stream>>>(
-            (const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k, pair_m, pair_n, ep);
+            (const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k, pair_m, pair_n, 1, ep);
         return hipGetLastError();
     }
     // Use the big tile once it alone can occupy every CU.
