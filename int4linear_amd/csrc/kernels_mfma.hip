@@ -581,6 +581,11 @@ constexpr int kPairStageBytes = 2 * kPairTile * kRowBytes;    // 16 KiB: X rows,
 constexpr int kPairLdsBytes = kPairStages * kPairStageBytes;  // 64 KiB, also the merge area
 constexpr int kPairRounds = 2;  // used up to this many tiles per CU (two workgroups fit a CU); measured: beyond, the 256 x 256 tiles win
 
+//
+// DEEP: the widening of a stage is interleaved with the MFMAs of the stage before it, from a
+// second set of widened operands (187 registers: one workgroup per CU); otherwise it follows
+// them (110 registers: two workgroups fit a CU, and their waves fill each other's gaps).
+template <bool DEEP>
 __global__ __launch_bounds__(512) void mfma_pair_kernel(const uint8_t *__restrict__ X,
                                                         const uint8_t *__restrict__ W,
                                                         int32_t *__restrict__ Y, int M, int N, int K,
@@ -648,47 +653,141 @@ __global__ __launch_bounds__(512) void mfma_pair_kernel(const uint8_t *__restric
             for (int t = 0; t < 16; ++t)
                 acc[i][j][t] = 0;
 
-    // The MFMAs of a stage are issued one iteration late, behind the LDS reads of the next
-    // stage, so that those reads (and the widening that waits for them) run in their shadow.
-    v4i xlo[2], xhi[2], wlo[2], whi[2];
-    auto multiply = [&]() {
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(xlo[j], wlo[i], acc[i][j], 0, 0, 0);
-                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(xhi[j], whi[i], acc[i][j], 0, 0, 0);
+    if constexpr (DEEP) {
+        // The MFMAs of a stage are issued one iteration late, between the LDS reads of the next
+        // stage and, slot by slot, the 48 vector operations that widen that stage's fragments:
+        // a wave issues in order, so widening done after the eight MFMAs would start only when the
+        // last of them has been issued, i.e. when the matrix pipe has nearly run dry.  The
+        // widened operands alternate between two register sets by the stage's parity; the four
+        // accumulators get their even-nibble MFMAs first, then the odd-nibble ones, so that no
+        // MFMA follows the one it depends on.
+        v4i xlo[2][2], xhi[2][2], wlo[2][2], whi[2][2];  // [parity of the stage][fragment]
+        auto arrive = [&](int st, v4i (&px)[2], v4i (&pw)[2]) {
+            // Stage st has landed once this wave's two loads of it have (the loads of the two
+            // younger stages may still be in flight) and every wave has said the same; by then
+            // every wave has also finished reading stage st - 1, whose buffer the loads of
+            // stage st + 3 now refill.
+            __builtin_amdgcn_s_waitcnt(I4L_VMCNT(2 * (kPairStages - 2)));
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            issue(st + kPairStages - 1);
+            const uint8_t *stage = lds + (st % kPairStages) * kPairStageBytes;
+    #pragma unroll
+            for (int j = 0; j < 2; ++j)
+                px[j] = *(const v4i *)(stage + x_rd + j * kFrag * kRowBytes);
+    #pragma unroll
+            for (int i = 0; i < 2; ++i)
+                pw[i] = *(const v4i *)(stage + w_rd + i * kFrag * kRowBytes);
+        };
+        // Operation op (0..47) of widening the four fragments of a stage into register set P:
+        // fragment op / 12 (X 0, X 1, W 0, W 1); within a fragment the four shifts, then the
+        // four masks of the shifted words, then the four masks of the unshifted words.
+        auto widen_op = [&](auto par_tag, int op, const v4i (&px)[2], const v4i (&pw)[2]) {
+            constexpr int P = decltype(par_tag)::value;
+            const int f = op / 12, k = op % 12, d = k % 4;
+            const v4i &src = f < 2 ? px[f] : pw[f - 2];
+            v4i &lo = f < 2 ? xlo[P][f] : wlo[P][f - 2];
+            v4i &hi = f < 2 ? xhi[P][f] : whi[P][f - 2];
+            if (k < 4)
+                lo[d] = src[d] << 4;
+            else if (k < 8)
+                lo[d] = lo[d] & himask;
+            else
+                hi[d] = src[d] & himask;
+        };
+        // MFMA `slot` (0..7) of the stage whose operands are in register set P.
+        auto mfma_slot = [&](auto par_tag, int slot) {
+            constexpr int P = decltype(par_tag)::value;
+            const int j = (slot >> 1) & 1, i = slot & 1;
+            if (slot < 4)
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(xlo[P][j], wlo[P][i], acc[i][j], 0, 0, 0);
+            else
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(xhi[P][j], whi[P][i], acc[i][j], 0, 0, 0);
+        };
+        // Stage st (parity P) arrives and is widened while stage st - 1 is multiplied.  The first
+        // two MFMAs go out bare (the LDS reads are still under way), the other six are each
+        // followed by eight of the widening operations.
+        auto body = [&](auto par_tag, int st) {
+            constexpr int P = decltype(par_tag)::value;
+            v4i px[2], pw[2];
+            arrive(st, px, pw);
+    #pragma unroll
+            for (int slot = 0; slot < 8; ++slot) {
+                mfma_slot(std::integral_constant<int, 1 - P>{}, slot);
+                if (slot >= 2) {
+    #pragma unroll
+                    for (int op = (slot - 2) * 8; op < (slot - 1) * 8; ++op)
+                        widen_op(par_tag, op, px, pw);
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
-    };
-#pragma unroll 1
-    for (int st = 0; st < KT; ++st) {
-        // Stage st has landed once this wave's two loads of it have (the loads of the two
-        // younger stages may still be in flight) and every wave has said the same; by then
-        // every wave has also finished reading stage st - 1, whose buffer the loads of
-        // stage st + 3 now refill.
-        __builtin_amdgcn_s_waitcnt(I4L_VMCNT(2 * (kPairStages - 2)));
-        __builtin_amdgcn_s_barrier();
-        asm volatile("" ::: "memory");
-        issue(st + kPairStages - 1);
-        const uint8_t *stage = lds + (st % kPairStages) * kPairStageBytes;
-        v4i px[2], pw[2];
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-            px[j] = *(const v4i *)(stage + x_rd + j * kFrag * kRowBytes);
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-            pw[i] = *(const v4i *)(stage + w_rd + i * kFrag * kRowBytes);
-        if (st > 0)
-            multiply();  // stage st - 1
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            xlo[j] = (px[j] << 4) & himask;
-            xhi[j] = px[j] & himask;
-            wlo[j] = (pw[j] << 4) & himask;
-            whi[j] = pw[j] & himask;
+        };
+        {
+            v4i px[2], pw[2];
+            arrive(0, px, pw);
+    #pragma unroll
+            for (int op = 0; op < 48; ++op)
+                widen_op(std::integral_constant<int, 0>{}, op, px, pw);
         }
+    #pragma unroll 1
+        for (int st = 1; st < KT; st += 2) {
+            body(std::integral_constant<int, 1>{}, st);
+            if (st + 1 < KT)
+                body(std::integral_constant<int, 0>{}, st + 1);
+        }
+        // the last stage
+        if ((KT - 1) & 1) {
+    #pragma unroll
+            for (int slot = 0; slot < 8; ++slot)
+                mfma_slot(std::integral_constant<int, 1>{}, slot);
+        } else {
+    #pragma unroll
+            for (int slot = 0; slot < 8; ++slot)
+                mfma_slot(std::integral_constant<int, 0>{}, slot);
+        }
+    } else {
+        // The MFMAs of a stage are issued one iteration late, behind the LDS reads of the next
+        // stage, so that those reads (and the widening that waits for them) run in their shadow.
+        v4i xlo[2], xhi[2], wlo[2], whi[2];
+        auto multiply = [&]() {
+    #pragma unroll
+            for (int j = 0; j < 2; ++j)
+    #pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(xlo[j], wlo[i], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(xhi[j], whi[i], acc[i][j], 0, 0, 0);
+                }
+        };
+    #pragma unroll 1
+        for (int st = 0; st < KT; ++st) {
+            // Stage st has landed once this wave's two loads of it have (the loads of the two
+            // younger stages may still be in flight) and every wave has said the same; by then
+            // every wave has also finished reading stage st - 1, whose buffer the loads of
+            // stage st + 3 now refill.
+            __builtin_amdgcn_s_waitcnt(I4L_VMCNT(2 * (kPairStages - 2)));
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            issue(st + kPairStages - 1);
+            const uint8_t *stage = lds + (st % kPairStages) * kPairStageBytes;
+            v4i px[2], pw[2];
+    #pragma unroll
+            for (int j = 0; j < 2; ++j)
+                px[j] = *(const v4i *)(stage + x_rd + j * kFrag * kRowBytes);
+    #pragma unroll
+            for (int i = 0; i < 2; ++i)
+                pw[i] = *(const v4i *)(stage + w_rd + i * kFrag * kRowBytes);
+            if (st > 0)
+                multiply();  // stage st - 1
+    #pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                xlo[j] = (px[j] << 4) & himask;
+                xhi[j] = px[j] & himask;
+                wlo[j] = (pw[j] << 4) & himask;
+                whi[j] = pw[j] & himask;
+            }
+        }
+        multiply();  // the last stage
     }
-    multiply();  // the last stage
 
     // ---- the upper group's sums go through LDS to the lower group, which stores the tile.
     //      Register r of lane l of quadrant q sits at word (q * 64 + r) * 64 + l.
@@ -865,8 +964,12 @@ hipError_t launch_mfma_splitk(const void *a, const void *b, void *c, int m, int 
         return launch_mfma(a, b, c, m, n, k, ep, dev, stream);
     // the K-slices run as work items of the small-grid form
     const int pair_m = (m + kPairTile - 1) / kPairTile, pair_n = (n + kPairTile - 1) / kPairTile;
-    mfma_pair_kernel<<<(unsigned)(pair_m * pair_n * d), 512, kPairLdsBytes, stream>>>(
-        (const uint8_t *)a, (const uint8_t *)b, (int32_t *)workspace, m, n, k, pair_m, pair_n, d, Epilogue{});
+    if ((long)pair_m * pair_n * d <= dev.cu_count)
+        mfma_pair_kernel<true><<<(unsigned)(pair_m * pair_n * d), 512, kPairLdsBytes, stream>>>(
+            (const uint8_t *)a, (const uint8_t *)b, (int32_t *)workspace, m, n, k, pair_m, pair_n, d, Epilogue{});
+    else
+        mfma_pair_kernel<false><<<(unsigned)(pair_m * pair_n * d), 512, kPairLdsBytes, stream>>>(
+            (const uint8_t *)a, (const uint8_t *)b, (int32_t *)workspace, m, n, k, pair_m, pair_n, d, Epilogue{});
     hipError_t e = hipGetLastError();
     if (e != hipSuccess)
         return e;
@@ -881,8 +984,12 @@ hipError_t launch_mfma(const void *a, const void *b, void *c, int m, int n, int 
     // Few 128 x 128 tiles per CU: the form whose two waves per SIMD split K.
     const int pair_m = (m + kPairTile - 1) / kPairTile, pair_n = (n + kPairTile - 1) / kPairTile;
     if ((long)pair_m * pair_n <= (long)dev.cu_count * kPairRounds) {
-        mfma_pair_kernel<<<(unsigned)(pair_m * pair_n), 512, kPairLdsBytes, stream>>>(
-            (const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k, pair_m, pair_n, 1, ep);
+        if ((long)pair_m * pair_n <= dev.cu_count)
+            mfma_pair_kernel<true><<<(unsigned)(pair_m * pair_n), 512, kPairLdsBytes, stream>>>(
+                (const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k, pair_m, pair_n, 1, ep);
+        else
+            mfma_pair_kernel<false><<<(unsigned)(pair_m * pair_n), 512, kPairLdsBytes, stream>>>(
+                (const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k, pair_m, pair_n, 1, ep);
         return hipGetLastError();
     }
     // Use the big tile once it alone can occupy every CU.
