@@ -860,6 +860,127 @@ __global__ __launch_bounds__(512) void mfma_pair_kernel(const uint8_t *__restric
     }
 }
 
+// The same form with a 64 x 64 tile, for grids so small that 128 x 128 tiles would leave
+// most CUs without one: wave w and wave w ^ 4 own the 32 x 32 quadrant w % 4 (one
+// accumulator fragment) and split every stage's K; a stage is 8 KiB, moved by one load per
+// wave (waves 0..3 the four chunks of X rows, waves 4..7 those of W rows).
+constexpr int kTinyTile = 64;
+constexpr int kTinyStageBytes = 2 * kTinyTile * kRowBytes;    // 8 KiB
+constexpr int kTinyLdsBytes = kPairStages * kTinyStageBytes;  // 32 KiB; the merge takes 16 KiB of it
+
+__global__ __launch_bounds__(512) void mfma_pair64_kernel(const uint8_t *__restrict__ X,
+                                                          const uint8_t *__restrict__ W,
+                                                          int32_t *__restrict__ Y, int M, int N, int K,
+                                                          int tiles_m, int tiles_n, Epilogue ep)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int half = wave >> 2;  // which half of every stage's K; also: 0 loads X, 1 loads W
+    const int quad = wave & 3;
+    const int wm = quad >> 1, wn = quad & 1;
+    const int rowbytes = K >> 1;
+    const int KT = K / kStageK;
+    int tm, tn;
+    tile_coords(blockIdx.x, tiles_m * tiles_n, tiles_m, tiles_n, tm, tn);
+    const int m0 = tm * kTinyTile, n0 = tn * kTinyTile;
+
+    // ---- loads: lane p of a chunk lands at byte 16 p: row p / 4, slot p % 4, and fetches the
+    //      row's chunk slot ^ swz(row).  Rows past the matrix re-read its last row.
+    const int ld_row = lane >> 2;
+    const int ld_c = (lane & 3) ^ swz(ld_row);
+    const int row_here = quad * kChunkRows + ld_row;
+    const int row = half ? min(row_here, N - 1 - n0) : min(row_here, M - 1 - m0);
+    const unsigned voff = (unsigned)row * (unsigned)rowbytes + (unsigned)ld_c * 16u;
+    const uint8_t *src_base = half ? W + (size_t)n0 * rowbytes : X + (size_t)m0 * rowbytes;
+    const unsigned lds_base = (unsigned)(size_t)I4L_LDS(lds);
+    const unsigned place = lds_base + (unsigned)(half * kTinyTile * kRowBytes + quad * kChunkBytes);
+    auto issue = [&](int st) {  // past the last stage the last one again, into a buffer nobody reads
+        const int src = st < KT ? st : KT - 1;
+        dma16(src_base + (size_t)src * kRowBytes, voff, place, (unsigned)((st % kPairStages) * kTinyStageBytes));
+    };
+#pragma unroll
+    for (int st = 0; st < kPairStages - 1; ++st)
+        issue(st);
+
+    const int fr = lane & 31;
+    const int fg = lane >> 5;
+    const unsigned rd_off = (unsigned)fr * kRowBytes + (unsigned)(((2 * half + fg) ^ swz(fr)) * 16);
+    const unsigned x_rd = (unsigned)(wm * kFrag * kRowBytes) + rd_off;
+    const unsigned w_rd = (unsigned)((kTinyTile + wn * kFrag) * kRowBytes) + rd_off;
+    const int himask = (int)0xF0F0F0F0u;
+    v16i acc;
+#pragma unroll
+    for (int t = 0; t < 16; ++t)
+        acc[t] = 0;
+    v4i xlo, xhi, wlo, whi;
+#pragma unroll 1
+    for (int st = 0; st < KT; ++st) {
+        // this wave's load of stage st has landed (two younger ones may be in flight), and
+        // after the barrier everybody's; the buffer of stage st - 1 is free for stage st + 3
+        __builtin_amdgcn_s_waitcnt(I4L_VMCNT(kPairStages - 2));
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        issue(st + kPairStages - 1);
+        const uint8_t *stage = lds + (st % kPairStages) * kTinyStageBytes;
+        const v4i px = *(const v4i *)(stage + x_rd);
+        const v4i pw = *(const v4i *)(stage + w_rd);
+        if (st > 0) {  // stage st - 1, behind the reads of stage st
+            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(xlo, wlo, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(xhi, whi, acc, 0, 0, 0);
+        }
+        xlo = (px << 4) & himask;
+        xhi = px & himask;
+        wlo = (pw << 4) & himask;
+        whi = pw & himask;
+    }
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(xlo, wlo, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(xhi, whi, acc, 0, 0, 0);
+
+    // ---- the upper group's sums go through LDS to the lower group, which stores the tile
+    __builtin_amdgcn_s_waitcnt(I4L_VMCNT(0));  // the loads past the end have landed too
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    int *merge = (int *)lds + (size_t)quad * 16 * 64 + lane;
+    if (half == 1) {
+#pragma unroll
+        for (int t = 0; t < 16; ++t)
+            merge[t * 64] = acc[t];
+    }
+    __syncthreads();
+    if (half == 1)
+        return;
+#pragma unroll
+    for (int t = 0; t < 16; ++t)
+        acc[t] = (acc[t] + merge[t * 64]) >> 8;  // both operands carried a factor 16
+    // accumulator t is  m = 8 (t / 4) + 4 (lane / 32) + t % 4,  n = lane % 32  of the quadrant
+    const int mw = m0 + wm * kFrag + 4 * (lane >> 5);
+    const int nw = n0 + wn * kFrag + (lane & 31);
+    int32_t *out = Y + (size_t)mw * N + nw;
+    if (!ep.bias && !ep.row_scale && !ep.col_scale && !ep.f32) {
+#pragma unroll
+        for (int t = 0; t < 16; ++t) {
+            const int dm = 8 * (t / 4) + (t % 4);
+            if (mw + dm < M && nw < N)
+                out[(size_t)dm * N] = acc[t];
+        }
+        return;
+    }
+    const int nn = min(nw, N - 1);
+    const int bias_v = ep.bias ? ep.bias[nn] : 0;
+    const float cs_v = ep.col_scale ? ep.col_scale[nn] : 1.f;
+    float rs[16];
+#pragma unroll
+    for (int t = 0; t < 16; ++t)
+        rs[t] = ep.row_scale ? ep.row_scale[min(mw + 8 * (t / 4) + (t % 4), M - 1)] : 1.f;
+#pragma unroll
+    for (int t = 0; t < 16; ++t) {
+        const int dm = 8 * (t / 4) + (t % 4);
+        if (mw + dm < M && nw < N)
+            out[(size_t)dm * N] = epilogue_value(ep, acc[t], bias_v, rs[t], cs_v);
+    }
+}
+
 // 256 x 256 tile, eight wavefronts of 128 (m) x 64 (n), one workgroup per CU, two
 // wavefronts per SIMD: the large-shape configuration.
 using CfgLarge = TileConfig<2, 4, 4, 2, 4, 1>;
@@ -923,10 +1044,11 @@ hipError_t launch_mfma_tile(const void *a, const void *b, void *c, int m, int n,
     return hipErrorInvalidValue;
 }
 
-// K-slices per tile for shapes whose 128 x 128 tiles would fill at most an eighth of the
-// device's 512 slots at K >= 4096, or less than a quarter of them at K >= 8192 (measured
-// against the unsplit small-grid form: with more tiles or shorter K the second pass over the
-// partial sums costs more than the idle CUs): the largest divisor of the stage count
+// K-slices per tile for shapes with few tiles and long K: at most a quarter as many 128 x 128
+// tiles as CUs at K >= 12288, or a sixteenth at K >= 8192 (measured against the unsplit
+// 64 x 64 form, which wins everywhere else: e.g. 160 x 4096 x 4096 9.6 against 16 us,
+// 1024 x 512 x 8192 16 against 20 us, but 128 x 4096 x 14336 26 against 19.5 us): the largest
+// divisor of the stage count
 // that keeps at least eight stages per slice, at most eight slices, and at most half a
 // work item per slot.
 int mfma_ksplit(int m, int n, int k, const DeviceInfo &dev)
@@ -936,8 +1058,8 @@ int mfma_ksplit(int m, int n, int k, const DeviceInfo &dev)
     const long tiles = (long)((m + CfgMedium::BM - 1) / CfgMedium::BM) * ((n + CfgMedium::BN - 1) / CfgMedium::BN);
     const long slots = (long)dev.cu_count * CfgMedium::OCC;
     const int stages = k / kStageK;
-    const bool few_tiles = tiles * 8 <= slots && stages >= 32;
-    const bool long_k = tiles * 4 < slots && stages >= 64;
+    const bool few_tiles = tiles * 16 <= dev.cu_count && stages >= 64;
+    const bool long_k = tiles * 4 <= dev.cu_count && stages >= 96;
     if (!few_tiles && !long_k)
         return 1;
     long limit = slots / (2 * tiles);
@@ -983,6 +1105,15 @@ hipError_t launch_mfma(const void *a, const void *b, void *c, int m, int n, int 
                              ((n + CfgLarge::BN - 1) / CfgLarge::BN);
     // Few 128 x 128 tiles per CU: the form whose two waves per SIMD split K.
     const int pair_m = (m + kPairTile - 1) / kPairTile, pair_n = (n + kPairTile - 1) / kPairTile;
+    // ... and so few that they would leave half of the CUs idle or more: 64 x 64 tiles
+    // (measured: 512 x 4096 x 4096 17 -> 14.5 us, 1024 x 1024 x 2048 10.8 -> 7.8 us; with more
+    // than cu_count / 2 tiles of 128 x 128 the larger tile wins).
+    if ((long)pair_m * pair_n * 2 <= dev.cu_count) {
+        const int tiny_m = (m + kTinyTile - 1) / kTinyTile, tiny_n = (n + kTinyTile - 1) / kTinyTile;
+        mfma_pair64_kernel<<<(unsigned)(tiny_m * tiny_n), 512, kTinyLdsBytes, stream>>>(
+            (const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k, tiny_m, tiny_n, ep);
+        return hipGetLastError();
+    }
     if ((long)pair_m * pair_n <= (long)dev.cu_count * kPairRounds) {
         if ((long)pair_m * pair_n <= dev.cu_count)
             mfma_pair_kernel<true><<<(unsigned)(pair_m * pair_n), 512, kPairLdsBytes, stream>>>(

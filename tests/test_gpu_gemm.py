@@ -248,11 +248,12 @@ def test_internal_workspace_shared_between_streams(gpu, host_threads):
 
 
 @pytest.mark.parametrize("m, n, k", [(128, 128, 128), (1, 1, 128), (129, 257, 384), (1000, 3000, 1024), (2048, 2048, 256),
-                                     (777, 1531, 2048), (2048, 4096, 512)])
+                                     (777, 1531, 2048), (2048, 4096, 512), (160, 4096, 4096), (300, 520, 4096), (65, 63, 1024)])
 def test_small_grid_form_of_the_int8_kernel(gpu, host_threads, m, n, k):
     """Up to two 128 x 128 tiles per CU the int8 kernel runs in the form whose two waves per
-    SIMD split every stage's K and merge their sums through LDS: plain and with every
-    epilogue, ragged edges in both directions, one to many stages."""
+    SIMD split every stage's K and merge their sums through LDS (with 64 x 64 tiles when the
+    larger ones would leave half of the CUs idle): plain and with every epilogue, ragged
+    edges in both directions, one to many stages."""
     import torch
 
     import int4linear_amd as lib
@@ -312,8 +313,8 @@ def test_split_k_form_of_the_fp6_kernel(gpu, host_threads, m, n, k):
     assert np.array_equal(yf.cpu().numpy().view(np.int32), oracle.epilogue(want, bias, rs, cs, f32=True).view(np.int32))
 
 
-@pytest.mark.parametrize("m, n, k", [(128, 4096, 14336), (160, 4096, 4096), (300, 520, 4096), (1024, 512, 8192),
-                                     (140, 1000, 4096), (200, 136, 16384)])
+@pytest.mark.parametrize("m, n, k", [(128, 4096, 14336), (300, 520, 12288), (1024, 512, 14336), (100, 300, 8192),
+                                     (140, 1000, 12288), (200, 136, 16384)])
 def test_split_k_form_of_the_int8_kernel(gpu, host_threads, m, n, k):
     """Few tiles and long K: automatic dispatch splits K over workgroups (partial sums in the
     internal workspace, a second kernel adds them and applies the epilogue)."""
