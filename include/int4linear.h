@@ -125,9 +125,7 @@ void int4linear_set_workspace_limit(size_t bytes);
 int int4linear_release_workspace(void);
 
 /* Name of the kernel INT4LINEAR_KERNEL_AUTO would pick for a shape ("simple", "mfma",
- * "fp6", "skinny"); never NULL.  For 65..128 rows of X the choice between "skinny" and
- * "mfma" depends on the current device's CU count, which is known after the first call
- * on that device (int4linear_init() counts); before that the answer is "mfma". */
+ * "fp6", "skinny"); never NULL. */
 const char *int4linear_kernel_for_shape(int m, int n, int k);
 
 /* Human-readable text for a status code; never NULL. */

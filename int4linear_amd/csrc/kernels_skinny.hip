@@ -1002,20 +1002,12 @@ bool skinny_supports(int m, int n, int k)
     return m <= kMaxRows && make_plan(m, n, k, 1, p);
 }
 
-// Where the kernel is the fastest one: up to 64 rows of X always; up to 128 when one
-// workgroup per CU covers W and K needs a single pass (W is then streamed twice, the
-// second time through the caches, which still beats 128 x 128 tiles that leave more
-// than half of the CUs idle).
-bool skinny_preferred(int m, int n, int k, const DeviceInfo &dev)
+// Where the kernel is the fastest one: up to 64 rows of X.  With more rows it takes X in runs
+// of 64 and streams W again for each (128 x 14336 x 4096: 21 us), which the int8 kernel's
+// small-grid forms beat from 65 rows on (17.7 us; 65 rows: 15.5 against 20 us).
+bool skinny_preferred(int m, int n, int k, const DeviceInfo &)
 {
-    if (!skinny_supports(m, n, k))
-        return false;
-    if (m <= 64)
-        return true;
-    Plan p;
-    if (m > 128 || dev.cu_count <= 0 || !make_plan(m, n, k, dev.cu_count, p))
-        return false;
-    return p.passes == 1 && (n + p.rows_blk - 1) / p.rows_blk <= dev.cu_count;
+    return m <= 64 && skinny_supports(m, n, k);
 }
 
 hipError_t launch_skinny(const void *a, const void *b, void *c, int m, int n, int k,

@@ -84,9 +84,8 @@ def test_kernel_dispatch_table():
     assert lib.kernel_for_shape(16, 4096, 4096) == "skinny"
     assert lib.kernel_for_shape(1, 14336, 4096) == "skinny"
     assert lib.kernel_for_shape(64, 4096, 14336) == "skinny"
-    # 65..128 rows: the weight-streaming kernel where one workgroup per CU covers W, which needs
-    # the device's CU count (unknown before the first call on a device: then the int8 kernel)
-    assert lib.kernel_for_shape(65, 4096, 4096) in ("mfma", "skinny")
+    # from 65 rows on the int8 kernel's small-grid forms are faster than runs of 64 rows
+    assert lib.kernel_for_shape(65, 4096, 4096) == "mfma"
     assert lib.kernel_for_shape(129, 4096, 4096) == "mfma"
     assert lib.kernel_for_shape(128, 128, 64) == "simple"     # K below one pipeline stage
     assert lib.kernel_for_shape(128, 128, 200) == "simple"    # K % 128 != 0, tiny
