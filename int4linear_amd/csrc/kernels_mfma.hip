@@ -1044,10 +1044,11 @@ hipError_t launch_mfma_tile(const void *a, const void *b, void *c, int m, int n,
     return hipErrorInvalidValue;
 }
 
-// K-slices per tile for shapes with few tiles and long K: at most a quarter as many 128 x 128
+// K-slices per tile for shapes with few tiles and long K: at most half as many 128 x 128
 // tiles as CUs at K >= 12288, or a sixteenth at K >= 8192 (measured against the unsplit
 // 64 x 64 form, which wins everywhere else: e.g. 160 x 4096 x 4096 9.6 against 16 us,
-// 1024 x 512 x 8192 16 against 20 us, but 128 x 4096 x 14336 26 against 19.5 us): the largest
+// 1024 x 512 x 8192 16 against 20 us, but 128 x 4096 x 14336 26 against 19.5 us and
+// 512 x 4096 x 14336 52 against 41 us): the largest
 // divisor of the stage count
 // that keeps at least eight stages per slice, at most eight slices, and at most half a
 // work item per slot.
@@ -1059,7 +1060,7 @@ int mfma_ksplit(int m, int n, int k, const DeviceInfo &dev)
     const long slots = (long)dev.cu_count * CfgMedium::OCC;
     const int stages = k / kStageK;
     const bool few_tiles = tiles * 16 <= dev.cu_count && stages >= 64;
-    const bool long_k = tiles * 4 <= dev.cu_count && stages >= 96;
+    const bool long_k = tiles * 2 <= dev.cu_count && stages >= 96;
     if (!few_tiles && !long_k)
         return 1;
     long limit = slots / (2 * tiles);
