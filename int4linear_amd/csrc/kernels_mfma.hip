@@ -871,7 +871,7 @@ constexpr int kTinyLdsBytes = kPairStages * kTinyStageBytes;  // 32 KiB; the mer
 __global__ __launch_bounds__(512) void mfma_pair64_kernel(const uint8_t *__restrict__ X,
                                                           const uint8_t *__restrict__ W,
                                                           int32_t *__restrict__ Y, int M, int N, int K,
-                                                          int tiles_m, int tiles_n, Epilogue ep)
+                                                          int tiles_m, int tiles_n, int ksplit, Epilogue ep)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int lane = threadIdx.x & 63;
@@ -880,10 +880,14 @@ __global__ __launch_bounds__(512) void mfma_pair64_kernel(const uint8_t *__restr
     const int quad = wave & 3;
     const int wm = quad >> 1, wn = quad & 1;
     const int rowbytes = K >> 1;
-    const int KT = K / kStageK;
+    // ksplit > 1: workgroup v is K-slice v / tiles of tile v % tiles, as in the larger form
+    const int tiles = tiles_m * tiles_n;
+    const int slice = blockIdx.x / tiles;
+    const int KT = K / kStageK / ksplit;
     int tm, tn;
-    tile_coords(blockIdx.x, tiles_m * tiles_n, tiles_m, tiles_n, tm, tn);
+    tile_coords(blockIdx.x - slice * tiles, tiles, tiles_m, tiles_n, tm, tn);
     const int m0 = tm * kTinyTile, n0 = tn * kTinyTile;
+    Y += (size_t)slice * (size_t)M * (size_t)N;
 
     // ---- loads: lane p of a chunk lands at byte 16 p: row p / 4, slot p % 4, and fetches the
     //      row's chunk slot ^ swz(row).  Rows past the matrix re-read its last row.
@@ -892,7 +896,7 @@ __global__ __launch_bounds__(512) void mfma_pair64_kernel(const uint8_t *__restr
     const int row_here = quad * kChunkRows + ld_row;
     const int row = half ? min(row_here, N - 1 - n0) : min(row_here, M - 1 - m0);
     const unsigned voff = (unsigned)row * (unsigned)rowbytes + (unsigned)ld_c * 16u;
-    const uint8_t *src_base = half ? W + (size_t)n0 * rowbytes : X + (size_t)m0 * rowbytes;
+    const uint8_t *src_base = (half ? W + (size_t)n0 * rowbytes : X + (size_t)m0 * rowbytes) + (size_t)slice * KT * kRowBytes;
     const unsigned lds_base = (unsigned)(size_t)I4L_LDS(lds);
     const unsigned place = lds_base + (unsigned)(half * kTinyTile * kRowBytes + quad * kChunkBytes);
     auto issue = [&](int st) {  // past the last stage the last one again, into a buffer nobody reads
@@ -957,7 +961,7 @@ __global__ __launch_bounds__(512) void mfma_pair64_kernel(const uint8_t *__restr
     const int mw = m0 + wm * kFrag + 4 * (lane >> 5);
     const int nw = n0 + wn * kFrag + (lane & 31);
     int32_t *out = Y + (size_t)mw * N + nw;
-    if (!ep.bias && !ep.row_scale && !ep.col_scale && !ep.f32) {
+    if (ksplit > 1 || (!ep.bias && !ep.row_scale && !ep.col_scale && !ep.f32)) {
 #pragma unroll
         for (int t = 0; t < 16; ++t) {
             const int dm = 8 * (t / 4) + (t % 4);
@@ -1087,6 +1091,23 @@ hipError_t launch_mfma_splitk(const void *a, const void *b, void *c, int m, int 
         return launch_mfma(a, b, c, m, n, k, ep, dev, stream);
     // the K-slices run as work items of the small-grid form
     const int pair_m = (m + kPairTile - 1) / kPairTile, pair_n = (n + kPairTile - 1) / kPairTile;
+    // With very few tiles (a sixteenth as many as CUs) the slices are 64 x 64 tiles, as many
+    // slices as leave at most two work items per CU (200 x 136 x 16384: 15.3 -> 11.6 us; with
+    // more tiles the 128 x 128 slices are as fast or faster).
+    if ((long)pair_m * pair_n * 16 <= dev.cu_count) {
+        const int tiny_m = (m + kTinyTile - 1) / kTinyTile, tiny_n = (n + kTinyTile - 1) / kTinyTile;
+        const int stages = k / kStageK;
+        int dt = 1;  // at most d: the slabs have room for d slices
+        for (int q = 2; q <= d; ++q)
+            if (stages % q == 0 && (long)tiny_m * tiny_n * q <= (long)dev.cu_count * 2)
+                dt = q;
+        mfma_pair64_kernel<<<(unsigned)(tiny_m * tiny_n * dt), 512, kTinyLdsBytes, stream>>>(
+            (const uint8_t *)a, (const uint8_t *)b, (int32_t *)workspace, m, n, k, tiny_m, tiny_n, dt, Epilogue{});
+        const hipError_t e2 = hipGetLastError();
+        if (e2 != hipSuccess)
+            return e2;
+        return launch_splitk_reduce(workspace, c, (size_t)m * (size_t)n, dt, n, ep, stream);
+    }
     if ((long)pair_m * pair_n * d <= dev.cu_count)
         mfma_pair_kernel<true><<<(unsigned)(pair_m * pair_n * d), 512, kPairLdsBytes, stream>>>(
             (const uint8_t *)a, (const uint8_t *)b, (int32_t *)workspace, m, n, k, pair_m, pair_n, d, Epilogue{});
@@ -1112,7 +1133,7 @@ hipError_t launch_mfma(const void *a, const void *b, void *c, int m, int n, int 
     if ((long)pair_m * pair_n * 2 <= dev.cu_count) {
         const int tiny_m = (m + kTinyTile - 1) / kTinyTile, tiny_n = (n + kTinyTile - 1) / kTinyTile;
         mfma_pair64_kernel<<<(unsigned)(tiny_m * tiny_n), 512, kTinyLdsBytes, stream>>>(
-            (const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k, tiny_m, tiny_n, ep);
+            (const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k, tiny_m, tiny_n, 1, ep);
         return hipGetLastError();
     }
     if ((long)pair_m * pair_n <= (long)dev.cu_count * kPairRounds) {
