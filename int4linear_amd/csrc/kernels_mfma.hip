@@ -23,6 +23,11 @@
 // the matrix pipe busy.  The kernel is persistent: gridDim.x workgroups walk a list of
 // tiles, and the load ring runs NSTAGE-1 stages ahead of the math ACROSS tile
 // boundaries, so the next tile's first stages are in flight while this tile stores C.
+//
+// Grids of few tiles run in a second form (mfma_pair_kernel, mfma_pair64_kernel: one
+// 128 x 128 or 64 x 64 tile per workgroup, eight waves of which the two on a SIMD split
+// every stage's K), described where it is defined; shapes with few tiles and long K are
+// split over K into slabs of partial sums that a second kernel adds up.
 #include "kernels.h"
 
 #include <type_traits>
