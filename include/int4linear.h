@@ -19,7 +19,10 @@
  * partial sums of either MFMA kernel's split-K form: created on first need, grown when a
  * larger problem arrives, never larger than the workspace limit, freed by
  * int4linear_release_workspace or at process exit.  With the limit set to 0 no entry
- * point allocates anything.
+ * point allocates anything.  A call whose stream is being captured into a HIP graph never
+ * touches that workspace either: under automatic dispatch it runs the kernels that need
+ * none, and an explicit INT4LINEAR_KERNEL_FP6 request returns INT4LINEAR_ERR_UNSUPPORTED
+ * (graphs that want the FP6 kernel use int4linear_gemm_fp6_converted on their own buffers).
  */
 #ifndef INT4LINEAR_H
 #define INT4LINEAR_H
@@ -70,7 +73,7 @@ int int4linear_init(void);
 int int4linear_gemm_s4s4s32(const void *a_packed_d, const void *b_packed_d, void *c_d,
                             int m, int n, int k, void *stream);
 
-/* Same as above with an explicit kernel choice (INT4LINEAR_KERNEL_*).  Returns
+/* Same as int4linear_gemm_s4s4s32 with an explicit kernel choice (INT4LINEAR_KERNEL_*).  Returns
  * INT4LINEAR_ERR_UNSUPPORTED when that kernel cannot run the shape. */
 int int4linear_gemm_s4s4s32_ex(const void *a_packed_d, const void *b_packed_d, void *c_d,
                                int m, int n, int k, int kernel, void *stream);
@@ -112,9 +115,8 @@ int int4linear_gemm_fp6_converted(const void *a_conv_d, const void *b_conv_d, vo
                                   int m, int n, int k, void *stream);
 
 /* Bytes of internal workspace INT4LINEAR_KERNEL_AUTO would use for a shape on the current
- * device (0 when the chosen kernel needs none; the split-K forms depend on the device's CU
- * count, so before the device's first call the int8 form reports 0 and the FP6 form the
- * converted operands alone). */
+ * device (0 when the chosen kernel needs none).  Sets the device up if that has not
+ * happened yet, so the answer does not depend on what was called before. */
 size_t int4linear_workspace_bytes(int m, int n, int k);
 
 /* Upper bound for the internal workspace (default 1 GiB).  Shapes that would need more,
@@ -124,8 +126,9 @@ void int4linear_set_workspace_limit(size_t bytes);
 /* Frees the current device's internal workspace (it is re-created on next need). */
 int int4linear_release_workspace(void);
 
-/* Name of the kernel INT4LINEAR_KERNEL_AUTO would pick for a shape ("simple", "mfma",
- * "fp6", "skinny"); never NULL. */
+/* Name of the kernel INT4LINEAR_KERNEL_AUTO would pick for a shape on the current device
+ * ("simple", "mfma", "fp6", "skinny"); never NULL.  Sets the device up like a compute call
+ * does; without a usable device the answer is the one that depends on the shape alone. */
 const char *int4linear_kernel_for_shape(int m, int n, int k);
 
 /* Human-readable text for a status code; never NULL. */

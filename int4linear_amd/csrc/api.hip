@@ -92,44 +92,63 @@ bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 // int8 kernel's small-grid form is as fast or faster there (64 tiles: 62 against 81 us at
 // K = 14336, 122 against 131 and 115 against 109 us at K = 28672), so the automatic choice
 // leaves those shapes to it.
-bool fp6_worthwhile(int m, int n, int k, const DeviceInfo &dev)
+bool fp6_worthwhile(int m, int n, int k, const DeviceInfo &dev, size_t limit)
 {
     const long tiles = (long)((m + 255) / 256) * ((n + 255) / 256);
     const bool pays = (tiles >= 128 && k >= 8192) || (tiles >= 144 && k >= 3072) || (tiles >= 384 && k >= 1024);
-    return pays && fp6_supports(m, n, k) && fp6_workspace_bytes(m, n, k, dev) <= g_workspace_limit.load();
+    return pays && fp6_supports(m, n, k) && fp6_workspace_bytes(m, n, k, dev) <= limit;
 }
 
 // K that is not a multiple of 128 fits neither the int8 nor the weight-streaming kernel,
 // but the FP6 converter pads K with zeros: beyond a few million multiply-adds that beats
 // the scalar kernel by orders of magnitude even for a handful of rows.
-bool fp6_for_ragged_k(int m, int n, int k, const DeviceInfo &dev)
+bool fp6_for_ragged_k(int m, int n, int k, const DeviceInfo &dev, size_t limit)
 {
     return (k % 128) != 0 && fp6_supports(m, n, k) && (double)m * n * k >= (double)(1 << 22) &&
-           fp6_workspace_bytes(m, n, k, dev) <= g_workspace_limit.load();
+           fp6_workspace_bytes(m, n, k, dev) <= limit;
 }
 
-// What is known of the current device: all zero before the first call on it.
+// The current device's record, set up if it has not been yet; without a usable device an
+// all-zero DeviceInfo (the shape-only answers of the queries below).
 DeviceInfo current_device_info()
 {
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+    PerDevice *pd = nullptr;
+    if (ensure_init(&pd) != INT4LINEAR_OK || !pd)
         return DeviceInfo{};
-    return g_devices[dev].info;
+    return pd->info;
 }
 
-// `dev` is the device the call runs on (cu_count 0 if it has not been set up yet: shapes
-// whose choice depends on the CU count then get the choice that does not).
-int pick_kernel(int m, int n, int k, const DeviceInfo &dev)
+// `limit`: the most workspace the chosen kernel may use.
+int pick_kernel(int m, int n, int k, const DeviceInfo &dev, size_t limit)
 {
     if (skinny_preferred(m, n, k, dev))
         return INT4LINEAR_KERNEL_SKINNY;
-    if (fp6_worthwhile(m, n, k, dev))
+    if (fp6_worthwhile(m, n, k, dev, limit))
         return INT4LINEAR_KERNEL_FP6;
     if (mfma_supports(m, n, k))
         return INT4LINEAR_KERNEL_MFMA;
-    if (fp6_for_ragged_k(m, n, k, dev))
+    if (fp6_for_ragged_k(m, n, k, dev, limit))
         return INT4LINEAR_KERNEL_FP6;
     return INT4LINEAR_KERNEL_SIMPLE;
+}
+
+// Where a call's workspace comes from.
+enum class Workspace {
+    Internal,  // the per-device buffer this library allocates and grows (acquire_workspace)
+    None       // none: only kernels that need no workspace
+};
+
+// True while `stream` records into a graph.  Allocating, freeing and recording events on
+// other streams are all off limits then, and so is baking the internal workspace's address
+// into a graph that may outlive it.  A query that fails counts as capturing.
+bool stream_is_capturing(hipStream_t stream)
+{
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
+        (void)hipGetLastError();
+        return true;
+    }
+    return status != hipStreamCaptureStatusNone;
 }
 
 // Hands out the device's internal workspace with at least `need` bytes for work about to be
@@ -185,27 +204,33 @@ int acquire_workspace(PerDevice *pd, size_t need, hipStream_t stream, void **out
     return INT4LINEAR_OK;
 }
 
-// The FP6 path on the internal workspace.
+// The FP6 path: converted operands (and split-K slabs) in the internal workspace.
 int run_fp6(PerDevice *pd, const void *a, const void *b, void *c, int m, int n, int k,
-            const Epilogue &ep, hipStream_t stream)
+            const Epilogue &ep, Workspace source, hipStream_t stream)
 {
+    const size_t need = fp6_workspace_bytes(m, n, k, pd->info);
+    hipError_t e;
+    if (source == Workspace::None || stream_is_capturing(stream))
+        return INT4LINEAR_ERR_UNSUPPORTED;
     std::lock_guard<std::mutex> lock(pd->ws_mutex);
     void *ws = nullptr;
-    const int st = acquire_workspace(pd, fp6_workspace_bytes(m, n, k, pd->info), stream, &ws);
+    const int st = acquire_workspace(pd, need, stream, &ws);
     if (st != INT4LINEAR_OK)
         return st;
-    const hipError_t e = launch_fp6(a, b, c, m, n, k, ws, ep, pd->info, stream);
+    e = launch_fp6(a, b, c, m, n, k, ws, ep, pd->info, stream);
     return e == hipSuccess ? INT4LINEAR_OK : fail_hip(e);
 }
 
 // The int8 kernel under automatic dispatch: split over K when that helps and the workspace
 // for the partial sums can be had, otherwise the plain kernel.
 int run_mfma_auto(PerDevice *pd, const void *a, const void *b, void *c, int m, int n, int k,
-                  const Epilogue &ep, hipStream_t stream)
+                  const Epilogue &ep, Workspace source, hipStream_t stream)
 {
     const size_t need = mfma_workspace_bytes(m, n, k, pd->info);
     hipError_t e;
     if (need == 0) {
+        e = launch_mfma(a, b, c, m, n, k, ep, pd->info, stream);
+    } else if (source == Workspace::None || stream_is_capturing(stream)) {
         e = launch_mfma(a, b, c, m, n, k, ep, pd->info, stream);
     } else {
         std::lock_guard<std::mutex> lock(pd->ws_mutex);
@@ -218,7 +243,7 @@ int run_mfma_auto(PerDevice *pd, const void *a, const void *b, void *c, int m, i
 }
 
 int gemm_impl(const void *a, const void *b, void *c, int m, int n, int k, int kernel,
-              void *stream_v, const Epilogue &ep = Epilogue{})
+              void *stream_v, const Epilogue &ep = Epilogue{}, Workspace source = Workspace::Internal)
 {
     if (m < 0 || n < 0 || k < 0 || (k % 8) != 0)
         return INT4LINEAR_ERR_SHAPE;
@@ -250,12 +275,17 @@ int gemm_impl(const void *a, const void *b, void *c, int m, int n, int k, int ke
     }
 
     const bool automatic = kernel == INT4LINEAR_KERNEL_AUTO;
-    if (automatic)
-        kernel = pick_kernel(m, n, k, pd->info);
+    if (automatic) {
+        // A stream under capture gets the kernels without workspace.
+        size_t limit = g_workspace_limit.load();
+        if (limit > 0 && stream_is_capturing(stream))
+            limit = 0;
+        kernel = pick_kernel(m, n, k, pd->info, limit);
+    }
     if (kernel == INT4LINEAR_KERNEL_FP6) {
         if (!fp6_supports(m, n, k))
             return INT4LINEAR_ERR_UNSUPPORTED;
-        const int st6 = run_fp6(pd, a, b, c, m, n, k, ep, stream);
+        const int st6 = run_fp6(pd, a, b, c, m, n, k, ep, source, stream);
         // Under automatic dispatch a workspace that cannot be had falls back to a kernel
         // that needs none.
         if (st6 == INT4LINEAR_OK || !automatic)
@@ -272,7 +302,7 @@ int gemm_impl(const void *a, const void *b, void *c, int m, int n, int k, int ke
         if (!mfma_supports(m, n, k))
             return INT4LINEAR_ERR_UNSUPPORTED;
         if (automatic)
-            return run_mfma_auto(pd, a, b, c, m, n, k, ep, stream);
+            return run_mfma_auto(pd, a, b, c, m, n, k, ep, source, stream);
         e = launch_mfma(a, b, c, m, n, k, ep, pd->info, stream);
         break;
     case INT4LINEAR_KERNEL_MFMA_128:
@@ -427,7 +457,7 @@ const char *int4linear_kernel_for_shape(int m, int n, int k)
 {
     if (m < 0 || n < 0 || k < 0 || (k % 8) != 0)
         return "invalid";
-    switch (pick_kernel(m, n, k, current_device_info())) {
+    switch (pick_kernel(m, n, k, current_device_info(), g_workspace_limit.load())) {
     case INT4LINEAR_KERNEL_SKINNY:
         return "skinny";
     case INT4LINEAR_KERNEL_FP6:
@@ -468,11 +498,11 @@ size_t int4linear_workspace_bytes(int m, int n, int k)
     if (m < 1 || n < 1 || k < 8 || (k % 8) != 0)
         return 0;
     const DeviceInfo info = current_device_info();
-    const int kernel = pick_kernel(m, n, k, info);
+    const int kernel = pick_kernel(m, n, k, info, g_workspace_limit.load());
     if (kernel == INT4LINEAR_KERNEL_FP6)
         return fp6_workspace_bytes(m, n, k, info);
     if (kernel == INT4LINEAR_KERNEL_MFMA) {
-        // the split-K form needs the device's CU count: 0 before the first call on a device
+        // the split-K form needs the device's CU count: unknown only without a device
         if (info.cu_count == 0)
             return 0;
         const size_t need = mfma_workspace_bytes(m, n, k, info);
@@ -517,19 +547,19 @@ namespace {
 
 // Kernel of each step of the version history for a shape; a step whose kernel cannot take
 // the shape falls back to the step before it.
-int version_kernel(int version, int m, int n, int k)
+int version_kernel(int version, int m, int n, int k, const DeviceInfo &info)
 {
     const bool int8_ok = mfma_supports(m, n, k);
     switch (version) {
     case 21:
         return INT4LINEAR_KERNEL_AUTO;
     case 20:
-        if (fp6_supports(m, n, k) && fp6_workspace_bytes(m, n, k, current_device_info()) <= g_workspace_limit.load() &&
-            !skinny_preferred(m, n, k, current_device_info()))
+        if (fp6_supports(m, n, k) && fp6_workspace_bytes(m, n, k, info) <= g_workspace_limit.load() &&
+            !skinny_preferred(m, n, k, info))
             return INT4LINEAR_KERNEL_FP6;
         [[fallthrough]];
     case 11:
-        if (skinny_preferred(m, n, k, current_device_info()))
+        if (skinny_preferred(m, n, k, info))
             return INT4LINEAR_KERNEL_SKINNY;
         [[fallthrough]];
     case 10:
@@ -546,8 +576,9 @@ int version_kernel(int version, int m, int n, int k)
 void launch_version(const char *name, int version, void *x, void *w, void *y, int m, int n, int k)
 {
     const bool valid = m >= 0 && n >= 0 && k >= 0 && (k % 8) == 0;
-    ensure_init(nullptr);  // the choice below may depend on the device; a failure is reported by the launch
-    launch_blocking(name, x, w, y, m, n, k, valid ? version_kernel(version, m, n, k) : INT4LINEAR_KERNEL_AUTO);
+    // The choice may depend on the device; a device that cannot be set up is reported by the launch.
+    const DeviceInfo info = current_device_info();
+    launch_blocking(name, x, w, y, m, n, k, valid ? version_kernel(version, m, n, k, info) : INT4LINEAR_KERNEL_AUTO);
 }
 
 }  // namespace

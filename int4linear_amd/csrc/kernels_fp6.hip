@@ -592,7 +592,10 @@ bool fp6_supports(int m, int n, int k)
 {
     // fp32 accumulation of products bounded by 64 stays exact while K * 64 < 2^24.  The
     // converter pads K to a multiple of 128 with zeros, so any K % 8 == 0 is fine.
-    return m >= 1 && n >= 1 && k >= 8 && k % 8 == 0 && k <= (1 << 18) - kStageK;
+    // Rows: the converter's grid (one y block per 32 rows of either operand) ends at 65535
+    // and the store addresses a tile's 256 rows of C with byte offsets below 2^30.
+    constexpr int kMaxRows = (1 << 20) - kTileRows;
+    return m >= 1 && n >= 1 && m <= kMaxRows && n <= kMaxRows && k >= 8 && k % 8 == 0 && k <= (1 << 18) - kStageK;
 }
 
 int fp6_ksplit(int m, int n, int k, const DeviceInfo &dev)

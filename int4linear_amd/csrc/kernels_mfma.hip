@@ -73,9 +73,7 @@ __device__ __forceinline__ int opaque(int v)
 // Marks a value as used (and possibly changed) at this point of the program.
 __device__ __forceinline__ void keep(v4i &v) { asm volatile("" : "+v"(v)); }
 
-#ifndef I4L_STORE_AUX
-#define I4L_STORE_AUX 2  // nt: C is written once and not read back by this kernel
-#endif
+constexpr int kStoreAux = 2;  // nt: C is written once and not read back by this kernel
 
 constexpr int kStageK = 128;                 // nibbles of K per pipeline stage
 constexpr int kRowBytes = kStageK / 2;       // bytes per LDS row (64)
@@ -521,7 +519,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
 #pragma unroll
                         for (int i = 0; i < C::FN; ++i) {
                             const int v = acc[i][j][t] >> 8;
-                            __builtin_amdgcn_raw_buffer_store_b32((unsigned)v, rsrc, row_off + col_off[i], 0, I4L_STORE_AUX);
+                            __builtin_amdgcn_raw_buffer_store_b32((unsigned)v, rsrc, row_off + col_off[i], 0, kStoreAux);
                         }
                     }
                 }
@@ -554,7 +552,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
 #pragma unroll
                         for (int i = 0; i < C::FN; ++i) {
                             const int v = epilogue_value(ep, acc[i][j][t] >> 8, bias_v[i], rs[t], cs_v[i]);
-                            __builtin_amdgcn_raw_buffer_store_b32((unsigned)v, rsrc, row_off + col_off[i], 0, I4L_STORE_AUX);
+                            __builtin_amdgcn_raw_buffer_store_b32((unsigned)v, rsrc, row_off + col_off[i], 0, kStoreAux);
                         }
                     }
                 }
@@ -1030,7 +1028,8 @@ bool mfma_supports(int m, int n, int k)
 {
     // K <= 131071 keeps 256 * (sum of products) inside int32; one LDS row per stage is
     // 128 nibbles.
-    return m >= 1 && n >= 1 && k >= kStageK && k % kStageK == 0 && k <= 131071 - 127;
+    // The store addresses a tile's rows of C (at most 256) with byte offsets below 2^30.
+    return m >= 1 && n >= 1 && n <= (1 << 20) && k >= kStageK && k % kStageK == 0 && k <= 131071 - 127;
 }
 
 hipError_t mfma_init(const DeviceInfo &dev)

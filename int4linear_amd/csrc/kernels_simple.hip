@@ -21,21 +21,22 @@ __device__ __forceinline__ int nibble_s4(uint32_t word, int slot)
 // LDS one 128-nibble chunk at a time.  test/test_correctness.cu:12-19 semantics.
 __global__ __launch_bounds__(kTile *kTile) void simple_gemm_kernel(
     const uint32_t *__restrict__ a, const uint32_t *__restrict__ b, int32_t *__restrict__ c,
-    int m, int n, int k_words, Epilogue ep)
+    int m, int n, int k_words, unsigned tile_row0, Epilogue ep)
 {
     __shared__ uint32_t a_lds[kTile][kChunkWords + 1];
     __shared__ uint32_t b_lds[kTile][kChunkWords + 1];
 
     const int tx = threadIdx.x % kTile;  // column of C inside the tile
     const int ty = threadIdx.x / kTile;  // row of C inside the tile
-    const long row = (long)blockIdx.y * kTile + ty;
+    const long tile_row = (long)tile_row0 + blockIdx.y;  // a launch covers at most 65535 tile rows
+    const long row = tile_row * kTile + ty;
     const long col = (long)blockIdx.x * kTile + tx;
 
     int acc = 0;
     for (int w0 = 0; w0 < k_words; w0 += kChunkWords) {
         // Thread (ty, tx) stages word tx of row ty of each operand tile.
         const int w = w0 + tx;
-        const long a_row = (long)blockIdx.y * kTile + ty;
+        const long a_row = tile_row * kTile + ty;
         const long b_row = (long)blockIdx.x * kTile + ty;
         a_lds[ty][tx] = (a_row < m && w < k_words) ? a[a_row * k_words + w] : 0u;
         b_lds[ty][tx] = (b_row < n && w < k_words) ? b[b_row * k_words + w] : 0u;
@@ -137,12 +138,18 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const int32_t *__res
 hipError_t launch_simple(const void *a, const void *b, void *c, int m, int n, int k,
                          const Epilogue &ep, hipStream_t stream)
 {
-    dim3 grid((n + kTile - 1) / kTile, (m + kTile - 1) / kTile);
-    if (grid.y > 65535u)
-        return hipErrorInvalidValue;
-    simple_gemm_kernel<<<grid, kTile * kTile, 0, stream>>>(
-        (const uint32_t *)a, (const uint32_t *)b, (int32_t *)c, m, n, k / 8, ep);
-    return hipGetLastError();
+    // The grid's y extent ends at 65535: more tile rows than that go out as several launches.
+    const unsigned tile_rows = (unsigned)((m + kTile - 1) / kTile);
+    for (unsigned row0 = 0; row0 < tile_rows; row0 += 65535u) {
+        const unsigned rows = tile_rows - row0 < 65535u ? tile_rows - row0 : 65535u;
+        const dim3 grid((n + kTile - 1) / kTile, rows);
+        simple_gemm_kernel<<<grid, kTile * kTile, 0, stream>>>(
+            (const uint32_t *)a, (const uint32_t *)b, (int32_t *)c, m, n, k / 8, row0, ep);
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess)
+            return e;
+    }
+    return hipSuccess;
 }
 
 hipError_t launch_pack(const int *src, int *dst, int m, int n, hipStream_t stream)

@@ -444,6 +444,52 @@ def test_hip_graph_capture_and_replay(gpu, host_threads):
         assert np.array_equal(ysk.cpu().numpy(), oracle.linear_ref(x2, w2, threads=host_threads)), f"skinny, replay {rep}"
 
 
+def test_automatic_dispatch_under_graph_capture(gpu):
+    """A call with automatic dispatch on a stream that is being captured must not touch the
+    internal workspace (no allocation, no free, no events on other streams, no workspace
+    address baked into the graph): shapes that would take the FP6 kernel or a split-K form
+    run on kernels that need none, and an explicit FP6 request is refused.  The workspace is
+    released between the replays, which would invalidate any pointer a graph had kept."""
+    import torch
+
+    import int4linear_amd as lib
+
+    shapes = [(2304, 4096, 3072), (128, 4096, 14336), (40, 56, 4104)]  # fp6, int8 split-K, fp6 (ragged K)
+    assert [lib.kernel_for_shape(*s) for s in shapes] == ["fp6", "mfma", "fp6"]
+    assert all(lib.workspace_bytes(*s) > 0 for s in shapes)
+    bufs = []
+    for (m, n, k) in shapes:
+        bufs.append((torch.zeros(m * k // 2, dtype=torch.uint8, device="cuda:0"),
+                     torch.zeros(n * k // 2, dtype=torch.uint8, device="cuda:0"),
+                     torch.zeros((m, n), dtype=torch.int32, device="cuda:0"),
+                     torch.zeros((m, n), dtype=torch.int32, device="cuda:0")))
+    lib.release_workspace()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for (m, n, k), (xd, wd, yd, _) in zip(shapes, bufs):
+            lib.gemm_s4s4s32(xd, wd, yd, m, n, k)
+        with pytest.raises(lib.Int4LinearError) as refused:
+            lib.gemm_s4s4s32(bufs[0][0], bufs[0][1], bufs[0][2], *shapes[0], kernel="fp6")
+    assert refused.value.status == 5
+    g = torch.Generator(device="cuda:0")
+    for rep in range(3):
+        g.manual_seed(4200 + rep)
+        for (xd, wd, yd, ref) in bufs:
+            xd.copy_(torch.randint(0, 256, xd.shape, dtype=torch.uint8, device="cuda:0", generator=g))
+            wd.copy_(torch.randint(0, 256, wd.shape, dtype=torch.uint8, device="cuda:0", generator=g))
+            yd.fill_(-1)
+        # eager calls of the same shapes in between: these do use (and regrow) the workspace
+        for (m, n, k), (xd, wd, _, ref) in zip(shapes, bufs):
+            lib.gemm_s4s4s32(xd, wd, ref, m, n, k)
+        torch.cuda.synchronize()
+        lib.release_workspace()
+        graph.replay()
+        torch.cuda.synchronize()
+        for shape, (_, _, yd, ref) in zip(shapes, bufs):
+            assert torch.equal(yd, ref), f"{shape}, replay {rep}"
+
+
 def _random_shapes(count, seed):
     rng = np.random.default_rng(seed)
     shapes = []
