@@ -22,7 +22,8 @@
  * point allocates anything.  A call whose stream is being captured into a HIP graph never
  * touches that workspace either: under automatic dispatch it runs the kernels that need
  * none, and an explicit INT4LINEAR_KERNEL_FP6 request returns INT4LINEAR_ERR_UNSUPPORTED
- * (graphs that want the FP6 kernel use int4linear_gemm_fp6_converted on their own buffers).
+ * (graphs that want the FP6 kernel use int4linear_gemm_fp6_converted on their own buffers,
+ * or int4linear_gemm_s4s4s32_static).
  */
 #ifndef INT4LINEAR_H
 #define INT4LINEAR_H
@@ -41,7 +42,9 @@ enum {
     INT4LINEAR_ERR_ALIGN = 3,       /* operand base not 16-byte aligned                  */
     INT4LINEAR_ERR_HIP = 4,         /* a HIP runtime call failed (see last_hip_error)    */
     INT4LINEAR_ERR_UNSUPPORTED = 5, /* the requested kernel cannot run this shape        */
-    INT4LINEAR_ERR_NO_DEVICE = 6    /* no gfx950 device is visible                       */
+    INT4LINEAR_ERR_NO_DEVICE = 6,   /* no gfx950 device is visible                       */
+    INT4LINEAR_ERR_SCRATCH = 7      /* int4linear_gemm_s4s4s32_static: the shape needs more
+                                       than INT4LINEAR_STATIC_SCRATCH_BYTES of scratch   */
 };
 
 /* Kernel selector for int4linear_gemm_s4s4s32_ex. */
@@ -72,6 +75,25 @@ int int4linear_init(void);
  * synchronisation, and the direct kernel launch of test/benchmark.cu:46-72. */
 int int4linear_gemm_s4s4s32(const void *a_packed_d, const void *b_packed_d, void *c_d,
                             int m, int n, int k, void *stream);
+
+/* int4linear_gemm_s4s4s32 for callers that cannot allocate device memory: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart
+ * in the reference (whose launcher needs no scratch memory, kernels/linear_v21.cu:9-49).
+ * Same arguments, same result, same choice of kernel as int4linear_gemm_s4s4s32 makes with
+ * an unlimited workspace, but where that entry point would use its allocated workspace (the
+ * FP6 kernel's converted operands, the partial sums of the split-K forms) this one uses a
+ * fixed array of INT4LINEAR_STATIC_SCRATCH_BYTES that is part of the library's device image:
+ * every device the library is initialised on holds one copy until the process ends.  The
+ * call allocates and frees nothing, records no events and takes no locks.  A shape whose
+ * kernel would need more scratch than the array holds is refused with
+ * INT4LINEAR_ERR_SCRATCH before anything is enqueued (at M = N = K the FP6 form fits up to
+ * 9216; use int4linear_gemm_s4s4s32_ex with INT4LINEAR_KERNEL_MFMA for larger problems, it
+ * needs no scratch at all).  All calls on one device share the one array and nothing orders
+ * them: calls whose execution may overlap on a device (different streams, graphs replayed
+ * concurrently) race on it; calls on one stream are ordered by the stream. */
+#define INT4LINEAR_STATIC_SCRATCH_BYTES (128u << 20)
+int int4linear_gemm_s4s4s32_static(const void *a_packed_d, const void *b_packed_d, void *c_d,
+                                   int m, int n, int k, void *stream);
 
 /* Same as int4linear_gemm_s4s4s32 with an explicit kernel choice (INT4LINEAR_KERNEL_*).  Returns
  * INT4LINEAR_ERR_UNSUPPORTED when that kernel cannot run the shape. */

@@ -9,6 +9,7 @@ from .api import (  # noqa: F401
     fp6_operand_bytes,
     gemm_fp6_converted,
     gemm_s4s4s32,
+    gemm_s4s4s32_static,
     init,
     kernel_for_shape,
     linear_f32,

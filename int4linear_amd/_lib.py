@@ -18,6 +18,7 @@ LIB_PATH = Path(os.environ.get("INT4LINEAR_LIBRARY") or
 C_ABI = [
     ("int4linear_init", c_int, []),
     ("int4linear_gemm_s4s4s32", c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    ("int4linear_gemm_s4s4s32_static", c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     ("int4linear_gemm_s4s4s32_ex", c_int,
      [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     ("int4linear_pack_s32_to_s4", c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),

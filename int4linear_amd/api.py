@@ -51,6 +51,19 @@ def gemm_s4s4s32(a_packed_d, b_packed_d, c_d, m: int, n: int, k: int, *, kernel:
     _lib.check(st)
 
 
+STATIC_SCRATCH_BYTES = 128 << 20  # INT4LINEAR_STATIC_SCRATCH_BYTES
+
+
+def gemm_s4s4s32_static(a_packed_d, b_packed_d, c_d, m: int, n: int, k: int, *, stream: int | None = None) -> None:
+    """gemm_s4s4s32 with automatic dispatch on the library's fixed scratch array: allocates
+    nothing; shapes that need more scratch than the array holds raise (status 7)."""
+    lib = _lib.load()
+    if stream is None:
+        stream = _current_stream()
+    _lib.check(lib.int4linear_gemm_s4s4s32_static(_ptr(a_packed_d), _ptr(b_packed_d), _ptr(c_d), m, n, k,
+                                                  ctypes.c_void_p(stream)))
+
+
 def linear_s32(x_packed_d, w_packed_d, bias_d, y_d, m: int, n: int, k: int, *, kernel: str = "auto",
                stream: int | None = None) -> None:
     """Y = X * W^T + bias (int32); bias_d may be None."""

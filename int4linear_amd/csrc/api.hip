@@ -13,11 +13,21 @@ using namespace int4linear;
 
 constexpr int kMaxDevices = 64;
 
+// Scratch memory of int4linear_gemm_s4s4s32_static: it stands where the other entry points
+// use the workspace they allocate (the FP6 kernel's converted operands, the partial sums of
+// the split-K forms).  One copy per device, at its own address on each, for as long as the
+// process lives.  In host code the name below is only a handle for hipGetSymbolAddress, not
+// a device address: ensure_init() asks for the address once per device and everything else
+// uses PerDevice::scratch.
+constexpr size_t kStaticScratchBytes = (size_t)INT4LINEAR_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 struct PerDevice {
     std::once_flag once;
     hipError_t init_error = hipSuccess;
     int status = INT4LINEAR_OK;
     DeviceInfo info;
+    void *scratch = nullptr;  // this device's copy of `scratch` (kStaticScratchBytes bytes)
     // Workspace of the FP6 path: grown on demand up to g_workspace_limit, kept until
     // int4linear_release_workspace() or process exit.  `ws_event` marks the end of the
     // last GEMM that used it, so a call on another stream can wait for it.
@@ -67,6 +77,8 @@ int ensure_init(PerDevice **out)
             err = fp6_init(pd.info);
         if (err == hipSuccess)
             err = skinny_init(pd.info);
+        if (err == hipSuccess)  // `dev` is current here: the address is this device's copy
+            err = hipGetSymbolAddress((void **)&pd.scratch, HIP_SYMBOL(scratch));
         if (err != hipSuccess) {
             pd.init_error = err;
             pd.status = INT4LINEAR_ERR_HIP;
@@ -135,6 +147,7 @@ int pick_kernel(int m, int n, int k, const DeviceInfo &dev, size_t limit)
 // Where a call's workspace comes from.
 enum class Workspace {
     Internal,  // the per-device buffer this library allocates and grows (acquire_workspace)
+    Static,    // the file-scope `scratch` array: nothing is allocated, the size is fixed
     None       // none: only kernels that need no workspace
 };
 
@@ -204,20 +217,27 @@ int acquire_workspace(PerDevice *pd, size_t need, hipStream_t stream, void **out
     return INT4LINEAR_OK;
 }
 
-// The FP6 path: converted operands (and split-K slabs) in the internal workspace.
+// The FP6 path: converted operands (and split-K slabs) in the internal workspace or in the
+// static scratch array.
 int run_fp6(PerDevice *pd, const void *a, const void *b, void *c, int m, int n, int k,
             const Epilogue &ep, Workspace source, hipStream_t stream)
 {
     const size_t need = fp6_workspace_bytes(m, n, k, pd->info);
     hipError_t e;
-    if (source == Workspace::None || stream_is_capturing(stream))
-        return INT4LINEAR_ERR_UNSUPPORTED;
-    std::lock_guard<std::mutex> lock(pd->ws_mutex);
-    void *ws = nullptr;
-    const int st = acquire_workspace(pd, need, stream, &ws);
-    if (st != INT4LINEAR_OK)
-        return st;
-    e = launch_fp6(a, b, c, m, n, k, ws, ep, pd->info, stream);
+    if (source == Workspace::Static) {
+        if (need > kStaticScratchBytes)
+            return INT4LINEAR_ERR_SCRATCH;
+        e = launch_fp6(a, b, c, m, n, k, pd->scratch, ep, pd->info, stream);
+    } else {
+        if (source == Workspace::None || stream_is_capturing(stream))
+            return INT4LINEAR_ERR_UNSUPPORTED;
+        std::lock_guard<std::mutex> lock(pd->ws_mutex);
+        void *ws = nullptr;
+        const int st = acquire_workspace(pd, need, stream, &ws);
+        if (st != INT4LINEAR_OK)
+            return st;
+        e = launch_fp6(a, b, c, m, n, k, ws, ep, pd->info, stream);
+    }
     return e == hipSuccess ? INT4LINEAR_OK : fail_hip(e);
 }
 
@@ -230,6 +250,10 @@ int run_mfma_auto(PerDevice *pd, const void *a, const void *b, void *c, int m, i
     hipError_t e;
     if (need == 0) {
         e = launch_mfma(a, b, c, m, n, k, ep, pd->info, stream);
+    } else if (source == Workspace::Static) {
+        if (need > kStaticScratchBytes)
+            return INT4LINEAR_ERR_SCRATCH;
+        e = launch_mfma_splitk(a, b, c, m, n, k, pd->scratch, ep, pd->info, stream);
     } else if (source == Workspace::None || stream_is_capturing(stream)) {
         e = launch_mfma(a, b, c, m, n, k, ep, pd->info, stream);
     } else {
@@ -276,9 +300,12 @@ int gemm_impl(const void *a, const void *b, void *c, int m, int n, int k, int ke
 
     const bool automatic = kernel == INT4LINEAR_KERNEL_AUTO;
     if (automatic) {
-        // A stream under capture gets the kernels without workspace.
+        // The static scratch entry chooses as if memory were no object and then refuses what
+        // does not fit its array; a stream under capture gets the kernels without workspace.
         size_t limit = g_workspace_limit.load();
-        if (limit > 0 && stream_is_capturing(stream))
+        if (source == Workspace::Static)
+            limit = SIZE_MAX;
+        else if (limit > 0 && stream_is_capturing(stream))
             limit = 0;
         kernel = pick_kernel(m, n, k, pd->info, limit);
     }
@@ -288,7 +315,7 @@ int gemm_impl(const void *a, const void *b, void *c, int m, int n, int k, int ke
         const int st6 = run_fp6(pd, a, b, c, m, n, k, ep, source, stream);
         // Under automatic dispatch a workspace that cannot be had falls back to a kernel
         // that needs none.
-        if (st6 == INT4LINEAR_OK || !automatic)
+        if (st6 == INT4LINEAR_OK || !automatic || source == Workspace::Static)
             return st6;
         kernel = mfma_supports(m, n, k) ? INT4LINEAR_KERNEL_MFMA : INT4LINEAR_KERNEL_SIMPLE;
     }
@@ -348,6 +375,13 @@ int int4linear_gemm_s4s4s32(const void *a_packed_d, const void *b_packed_d, void
                             int n, int k, void *stream)
 {
     return gemm_impl(a_packed_d, b_packed_d, c_d, m, n, k, INT4LINEAR_KERNEL_AUTO, stream);
+}
+
+int int4linear_gemm_s4s4s32_static(const void *a_packed_d, const void *b_packed_d, void *c_d, int m,
+                                   int n, int k, void *stream)
+{
+    return gemm_impl(a_packed_d, b_packed_d, c_d, m, n, k, INT4LINEAR_KERNEL_AUTO, stream, Epilogue{},
+                     Workspace::Static);
 }
 
 int int4linear_gemm_s4s4s32_ex(const void *a_packed_d, const void *b_packed_d, void *c_d, int m,
@@ -486,6 +520,8 @@ const char *int4linear_status_string(int status)
         return "requested kernel does not support this shape";
     case INT4LINEAR_ERR_NO_DEVICE:
         return "no usable HIP device";
+    case INT4LINEAR_ERR_SCRATCH:
+        return "shape needs more scratch memory than the static array of int4linear_gemm_s4s4s32_static holds";
     default:
         return "unknown status";
     }
