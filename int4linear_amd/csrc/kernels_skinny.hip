@@ -1,30 +1,39 @@
 // Weight-streaming kernels for skinny M: the decode-shaped linear layer.  Three kernels:
-// skinny_kernel (up to 64 rows of X per run, W's rows split over one workgroup per CU and
-// per 64 rows), skinny_stream_kernel (very many rows of W: workgroups that stay on their
+// skinny_kernel (up to 64 rows of X per launch, W's rows split over one workgroup per CU),
+// skinny_stream_kernel (very many rows of W: workgroups that stay on their
 // CU) and skinny_basic_kernel (K that is not a whole number
 // of 128-byte tiles).
 //
 // The job is HBM-bound: every byte of W (N x K/2) is read exactly once and the arithmetic
 // (v_mfma_i32_16x16x64_i8 after the same 16x nibble widening as the big int8 kernel:
 // (w << 4) & 0xF0F0F0F0 and w & 0xF0F0F0F0, C = acc >> 8) is free next to it.  What decides
-// the speed is the shape of the global reads.  Measured on MI355X for a 28 MiB weight
-// matrix: a wave instruction whose eight-lane groups each read one whole 128-byte line
-// streams as fast as a plain linear read, while the natural MFMA pattern (sixteen rows,
-// 64 bytes of each) is 25 % slower.  So W is not loaded in MFMA layout.  Each load
+// the speed is the shape of the global reads and what a launch spends before its first load
+// and after its last byte.  Measured on MI355X for a 28 MiB weight matrix: a wave
+// instruction whose eight-lane groups each read one whole 128-byte line streams as fast as
+// a plain linear read, while the natural MFMA pattern (sixteen rows, 64 bytes of each) is
+// 25 % slower.  So W is not loaded in MFMA layout.  Each load
 // instruction moves eight rows x 128 bytes straight into LDS (global_load_lds_dwordx4,
 // non-temporal), and the MFMA operands are read back from LDS in fragment layout; a
 // 16-byte XOR swizzle of the slot index (applied by permuting which global chunk a lane
 // fetches, since the LDS position of a lane's data is fixed) keeps those reads free of
-// bank conflicts.
+// bank conflicts.  A lone wave issues an instruction only every five to seven cycles, so
+// every instruction between the wave's start and its first load, and between its last byte
+// and its store, is time nothing overlaps: 128 scalar instructions in front of the loads of
+// a bare streaming kernel cost 0.45 us per launch.  Hence the first loads go out after some
+// thirty instructions, the kernel arguments they need arrive preloaded in scalar registers
+// (the compile option -amdgpu-kernarg-preload-count), and the plain store path is a dozen
+// instructions.
 //
 // The rows of W are split evenly over the CUs in steps of eight; a workgroup holds its
 // rows as R groups of 16 (the last one possibly half empty) over the whole of K.  Its S
 // wavefronts split K into S slices of T tiles of 256 nibbles; a wave issues every load
 // of its slices before it waits for anything, multiplies each row group as soon as it has
 // landed (loads complete in issue order, so that is a wait for a known number of younger
-// loads), and the S partial sums meet once in LDS.  Each wave fetches its own slice of X
-// once and reuses it for its R row groups, so larger R cuts the (L2-resident, but
-// hot-line) X traffic.  No atomics, no workspace, and the result does not depend on timing.
+// loads), adds its share to the group's block of sums in LDS and counts itself in at the
+// group's arrival counter; the wave that completes a counter stores the group.  Each wave
+// fetches its own slice of X once and reuses it for its R row groups, so larger R cuts the
+// (L2-resident, but hot-line) X traffic.  No global atomics, no workspace, and the result
+// does not depend on timing (integer additions commute).
 #include "kernels.h"
 
 #include <utility>
@@ -64,6 +73,34 @@ __device__ __forceinline__ void dma16(const void *base, unsigned lane_off, unsig
                      :
                      : "v"(lane_off), "s"(base), "s"(lds_addr), "n"(IMM)
                      : "memory");
+}
+
+// The same with the LDS address given as a wave-uniform base plus the constant LDS_OFF: one
+// scalar addition straight into M0 instead of a precomputed address per load.
+template <bool NT, int IMM, int LDS_OFF>
+__device__ __forceinline__ void dma16_at(const void *base, unsigned lane_off, unsigned lds_base)
+{
+    static_assert(IMM >= 0 && IMM < 4096, "13-bit signed immediate");
+    static_assert(LDS_OFF - IMM >= 0, "the LDS base must not go below zero");
+    if (NT)
+        asm volatile("s_add_u32 m0, %2, %4\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%3 nt"
+                     :
+                     : "v"(lane_off), "s"(base), "s"(lds_base), "n"(IMM), "n"(LDS_OFF - IMM)
+                     : "memory", "scc");
+    else
+        asm volatile("s_add_u32 m0, %2, %4\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%3"
+                     :
+                     : "v"(lane_off), "s"(base), "s"(lds_base), "n"(IMM), "n"(LDS_OFF - IMM)
+                     : "memory", "scc");
+}
+
+// A wave-uniform value the compiler may have chosen to compute on the vector side: back into
+// scalar registers (the "s" operands of the load instructions need that).
+__device__ __forceinline__ unsigned uniform(unsigned v) { return (unsigned)__builtin_amdgcn_readfirstlane((int)v); }
+__device__ __forceinline__ const uint8_t *uniform(const uint8_t *p)
+{
+    const unsigned long long v = (unsigned long long)p;
+    return (const uint8_t *)((unsigned long long)uniform((unsigned)v) | ((unsigned long long)uniform((unsigned)(v >> 32)) << 32));
 }
 
 // f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>)
@@ -131,35 +168,60 @@ constexpr int max_threads(int t, int r, int fmx, bool xdma)
     return (!xdma && (t * fmx > 4 || (t * fmx == 4 && r * fmx >= 8))) ? 512 : 1024;
 }
 
+// LDS in front of the waves' tiles: the arrival counters, one per row group of W, in the first
+// 16 bytes (ds_append addresses them with the instruction's 16-bit constant), and from 1 KiB
+// on one 16 x 16 block of sums (1 KiB) per pair (row group of W, row group of X).
+constexpr int head_bytes(int r, int fmx) { return 1024 + r * fmx * 1024; }
+
 // T tiles per wave, R row groups per workgroup, FMX 16-row groups of X (M <= 16*FMX).
 // XDMA: X tiles go through LDS like W; otherwise they are loaded into registers in
 // fragment layout (for K so long that X tiles do not fit in LDS next to the W staging).
 //
 // A workgroup owns rows [blockIdx.x * rows_blk, + rows_blk) of W, rows_blk a multiple of 8
-// and at most 16*R.  Every wave issues all its loads up front in the order X, then row
-// group 0, 1, ...; since loads complete in order, "row group rg, tile t has landed" is a
-// wait for a fixed number of younger loads.  Each row group is multiplied, reduced across
-// the waves and stored as soon as it has landed, while the later groups are still in
-// flight, so only the last group's reduction is exposed after the last byte arrives.
+// and at most 16*R.  Every wave issues all its loads up front in the order first tile of W,
+// X, rest of W; since loads complete in order, "row group rg, tile t has landed" is a wait
+// for a fixed number of younger loads.  Each row group is multiplied and added to the
+// group's sums as soon as it has landed, while the later groups are still in flight, so
+// only the last group's share is exposed after the last byte arrives.
 template <int T, int R, int FMX, bool XDMA, bool RAGGED>
-__global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(const uint8_t *__restrict__ X_all,
-                                                      const uint8_t *__restrict__ W,
-                                                      int32_t *__restrict__ Y_all, int M_all, int N, int K,
-                                                      int rows_blk, int passes, Epilogue ep_all)
+__global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(const uint8_t *X, const uint8_t *W, int32_t *Y,
+                                                                              int M, int N, int K, int rows_blk, int passes,
+                                                                              int waves, Epilogue ep_all)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int kWaveTiles = T * (R + (XDMA ? FMX : 0));
+    constexpr int kHead = head_bytes(R, FMX);
 
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int waves = blockDim.x >> 6;  // S
-    const int rowbytes = K >> 1;
-    const int n0 = blockIdx.x * rows_blk;
-    const int n_end = min(N, n0 + rows_blk);  // > n0
+    // ---- first of all, the wave's first two loads (tile 0 of row group 0, first pass).
+    //      Nothing overlaps the time before a wave's first load, so these go out after as few
+    //      instructions as it takes; the values everything else is computed from pass through
+    //      an empty asm statement afterwards, which keeps the compiler from moving that work
+    //      up here.
+    int lane = threadIdx.x & 63;
+    int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    unsigned rowbytes = (unsigned)K >> 1;
+    int n0 = blockIdx.x * rows_blk;
+    int rows_here = min(rows_blk, N - n0);  // >= 1
     const unsigned lds_base = (unsigned)(size_t)I4L_LDS(lds);
-    const unsigned my_lds = lds_base + wave * kWaveTiles * kTileBytes;
+    {
+        // Lane p of a direct-to-LDS instruction lands at 16*p: tile row p/8 (+8 for the second
+        // instruction of a tile), slot p%8, so it fetches chunk slot ^ swizzle.
+        const unsigned lrow = (unsigned)lane >> 3, c8 = (unsigned)lane & 7;
+        const unsigned lim = (unsigned)min(rows_here - 1, 15);
+        const int skip0 = RAGGED ? max(0, (wave + 1) * T - K / kTileK) : 0;
+        const uint8_t *base = W + (size_t)n0 * rowbytes + (size_t)(wave * T - skip0) * kTileRowBytes;
+        const unsigned first_lds = lds_base + kHead + wave * kWaveTiles * kTileBytes;
+        dma16_at<true, 0, 0>(base, (unsigned)__umul24(min(lrow, lim), rowbytes) + ((c8 ^ (lrow >> 1)) << 4), first_lds);
+        dma16_at<true, 0, 1024>(base, (unsigned)__umul24(min(lrow + 8, lim), rowbytes) + ((c8 ^ (4 + (lrow >> 1))) << 4),
+                                first_lds);
+    }
+    asm volatile("" : "+v"(lane), "+s"(wave), "+s"(rowbytes), "+s"(n0), "+s"(rows_here), "+s"(M), "+s"(passes));
+
+    const unsigned my_lds = uniform(lds_base + kHead + wave * kWaveTiles * kTileBytes);
     const int himask = (int)0xF0F0F0F0u;
-    const uint8_t *mine = lds + wave * kWaveTiles * kTileBytes;
+    const uint8_t *mine = lds + kHead + wave * kWaveTiles * kTileBytes;
+    int *const arrived = (int *)lds;
+    int *const sums = (int *)(lds + 1024);
 
     // Fragment layout: lane l supplies row l%16 and, in step s of a tile, chunk
     // 4*s + l/16 (32 nibbles: even ones feed one MFMA, odd ones the next).
@@ -167,27 +229,6 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
     const int fg = lane >> 4;
     const int sw = slot_swizzle(fr);
 
-    // More than 16 * FMX rows of X are taken in runs of that many, one after the other: the
-    // workgroup's rows of W are then streamed again, from the caches they were just pulled
-    // through.
-#pragma unroll 1
-    for (int m_first = 0; m_first < M_all; m_first += 16 * FMX) {
-    const uint8_t *X = X_all + (size_t)m_first * rowbytes;
-    int32_t *Y = Y_all + (size_t)m_first * N;
-    const int M = min(M_all - m_first, 16 * FMX);
-    Epilogue ep = ep_all;
-    if (ep.row_scale)
-        ep.row_scale += m_first;
-
-    // ---- loads.  Lane p of a direct-to-LDS instruction lands at 16*p: tile row p/8 (+8
-    //      for the second instruction of a tile), slot p%8, so it fetches chunk
-    //      slot ^ swizzle.  Rows past the workgroup's (or the matrix's) end re-read the
-    //      last valid row: every wave issues the same number of loads, which the waits
-    //      below rely on, and nothing is read out of bounds.
-    //
-    // K longer than S * T tiles is covered in several passes: pass c takes the c-th run of
-    // S * T tiles, each wave refills its own LDS tiles (nobody else reads them, and its own
-    // reads of the previous pass have been consumed) and keeps accumulating.
     // With X in registers and an even T the X loads are made in a form the memory pipeline
     // takes at full rate (every quad of lanes reads 64 contiguous bytes of one row; the
     // fragment form, in which neighbouring lanes read different rows, is served at less
@@ -195,240 +236,278 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
     // Over a pair of tiles (256 bytes of a row, chunks 0..15) register j of the pair then
     // holds, for lane (fr, fg), chunk 4 * fg + j of row fr, and W is read from LDS to match.
     constexpr bool kPairX = !XDMA && T % 2 == 0;
-    // Row groups of W issued before X: the weight stream starts at once, X follows.
-    constexpr int kGroupsBeforeX = (!XDMA && R > 1) ? 1 : 0;
-    // With a single row group its first tile goes out before X for the same reason (the
-    // waits below need no change: X then sits right behind that tile).
-    constexpr int kTilesBeforeX = (!XDMA && R == 1 && T > 1) ? 1 : 0;
     v4i xg[XDMA ? 1 : T][2][FMX];
-    v4i acc[R][FMX];
-#pragma unroll
-    for (int rg = 0; rg < R; ++rg)
-#pragma unroll
-        for (int f = 0; f < FMX; ++f)
-            acc[rg][f] = (v4i){0, 0, 0, 0};
 
+    // K longer than S * T tiles is covered in several passes: pass c takes the c-th run of
+    // S * T tiles, each wave refills its own LDS tiles (nobody else reads them, and its own
+    // reads of the previous pass have been consumed).
     int skip = 0;
+    unsigned to_store = 0;  // row groups this wave was the last to arrive at
 #pragma unroll 1
     for (int pass = 0; pass < passes; ++pass) {
     {
-    // Per-lane byte offsets of the loads, relative to the wave's slice of the workgroup's
-    // first row of W, or of row 0 of X.
-    // (Derived anew in every pass from a copy of the lane number that the compiler cannot
-    // see through: kept across the multiplication they would cost registers there.)
+    // ---- loads.  Rows past the workgroup's (or the matrix's) end re-read the last valid
+    //      row: every wave issues the same number of loads, which the waits below rely on,
+    //      and nothing is read out of bounds.
+    // (The offsets are derived anew in every pass from a copy of the lane number that the
+    // compiler cannot see through: kept across the multiplication they would cost registers
+    // there.)
     int lane_here = lane;
     asm volatile("" : "+v"(lane_here));
-    const int lrow = lane_here >> 3;
+    const unsigned lrow = (unsigned)lane_here >> 3;
+    const unsigned c8 = (unsigned)lane_here & 7;
+    const unsigned chunk[2] = {(c8 ^ (lrow >> 1)) << 4, (c8 ^ (4 + (lrow >> 1))) << 4};
+    // This wave's slice of every row: T tiles from tile (pass * S + wave) * T on.  When
+    // K's tiles do not fill the last slices, a slice that would run past the end is
+    // moved back to end with the last tile, and its first `skip` tiles (someone else's,
+    // or all T of them) are loaded like the others but not multiplied.
+    const int first_tile = (pass * waves + wave) * T;
+    if (RAGGED)
+        skip = max(0, first_tile + T - K / kTileK);
+    const size_t kbyte0 = (size_t)(first_tile - skip) * kTileRowBytes;
+    const uint8_t *wbase = uniform(W + (size_t)n0 * rowbytes + kbyte0);
     unsigned w_off[R][2];
 #pragma unroll
     for (int rg = 0; rg < R; ++rg)
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            const int wr = rg * 16 + lrow + 8 * u;
-            w_off[rg][u] = (unsigned)(wr < n_end - n0 ? wr : n_end - n0 - 1) * rowbytes +
-                           ((lane_here & 7) ^ slot_swizzle(lrow + 8 * u)) * 16;
-        }
+        for (int u = 0; u < 2; ++u)
+            w_off[rg][u] = (unsigned)__umul24(min(16 * rg + lrow + 8 * u, (unsigned)(rows_here - 1)), rowbytes) + chunk[u];
+    auto issue_w = [&](auto rgc, auto first, auto count) {  // tiles first .. first + count - 1 of group rg
+        constexpr int rg = decltype(rgc)::value;
+        static_for<count()>([&](auto i) {
+            constexpr int t = first() + i();
+            dma16_at<true, t * kTileRowBytes, (rg * T + t) * kTileBytes>(wbase, w_off[rg][0], my_lds);
+            dma16_at<true, t * kTileRowBytes, (rg * T + t) * kTileBytes + 1024>(wbase, w_off[rg][1], my_lds);
+        });
+    };
+    constexpr std::integral_constant<int, 0> kZero{};
+    constexpr std::integral_constant<int, 1> kOne{};
+    constexpr std::integral_constant<int, T - 1> kRestOfGroup{};
+    constexpr std::integral_constant<int, T> kAllTiles{};
+    // Issue order: the first tile of W (in the first pass it is on its way already), X, the
+    // rest of W.
+    if (pass > 0)
+        issue_w(kZero, kZero, kOne);
+    // With the first loads on their way: the arrival counters and the sums start at zero,
+    // which everybody has to have seen before anybody adds to them.  (Meeting here, where
+    // every wave is about to wait for memory anyway, measured better than meeting in front
+    // of the first addition.)
+    if (pass == 0) {
+        if (threadIdx.x < 4)
+            arrived[threadIdx.x] = 0;
+        for (int i = threadIdx.x; i < R * FMX * 256; i += waves * 64)
+            sums[i] = 0;
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    }
     // X: through LDS like W (two loads per tile); as fragments (row fr, 64 bytes of a tile
     // per load); or in the paired form, where load j of a tile pair has quad q read row
     // 4 * (q % 4) + j, bytes 64 * (q / 4) .. + 64 of the pair.
-    constexpr int kXPatterns = XDMA ? 2 : kPairX ? 4 : 1;
-    unsigned x_off[FMX][kXPatterns];
-#pragma unroll
-    for (int f = 0; f < FMX; ++f)
-#pragma unroll
-        for (int j = 0; j < kXPatterns; ++j) {
-            const int q = lane_here >> 2;
-            const int xr = f * 16 + (XDMA ? lrow + 8 * j : kPairX ? 4 * (q & 3) + j : (lane_here & 15));
-            const int within = XDMA ? ((lane_here & 7) ^ slot_swizzle(lrow + 8 * j)) * 16
-                               : kPairX ? 64 * (q >> 2) + 16 * (lane_here & 3) : (lane_here >> 4) * 16;
-            x_off[f][j] = (unsigned)(xr < M ? xr : M - 1) * rowbytes + within;
-        }
-        // This wave's slice of every row: T tiles from tile (pass * S + wave) * T on.  When
-        // K's tiles do not fill the last slices, a slice that would run past the end is
-        // moved back to end with the last tile, and its first `skip` tiles (someone else's,
-        // or all T of them) are loaded like the others but not multiplied.
-        const int first_tile = (pass * waves + wave) * T;
-        if (RAGGED)
-            skip = max(0, first_tile + T - K / kTileK);
-        const size_t kbyte0 = (size_t)(first_tile - skip) * kTileRowBytes;
-        const uint8_t *wbase = W + (size_t)n0 * rowbytes + kbyte0;
-        const uint8_t *xbase = X + kbyte0;
-        auto issue_w = [&](int rg, auto first, auto count) {  // tiles first .. first + count - 1 of group rg
-            static_for<count()>([&](auto i) {
-                constexpr int t = first() + i();
-#pragma unroll
-                for (int u = 0; u < 2; ++u)
-                    dma16<true, t * kTileRowBytes>(wbase, w_off[rg][u], my_lds + (rg * T + t) * kTileBytes + u * 1024);
-            });
-        };
-        constexpr std::integral_constant<int, 0> kZero{};
-        constexpr std::integral_constant<int, T> kAllTiles{};
-        constexpr std::integral_constant<int, kTilesBeforeX> kHead{};
-        constexpr std::integral_constant<int, T - kTilesBeforeX> kTail{};
-#pragma unroll
-        for (int rg = 0; rg < kGroupsBeforeX; ++rg)
-            issue_w(rg, kZero, kAllTiles);
-        if constexpr (kTilesBeforeX > 0)
-            issue_w(0, kZero, kHead);
+    {
+        const uint8_t *xbase = uniform(X + kbyte0);
+        constexpr int kXPatterns = XDMA ? 2 : kPairX ? 4 : 1;
 #pragma unroll
         for (int f = 0; f < FMX; ++f) {
+            unsigned x_off[kXPatterns];
+#pragma unroll
+            for (int j = 0; j < kXPatterns; ++j) {
+                const unsigned q = (unsigned)lane_here >> 2;
+                const unsigned xr = f * 16 + (XDMA ? lrow + 8 * j : kPairX ? 4 * (q & 3) + j : ((unsigned)lane_here & 15));
+                const unsigned within = XDMA ? chunk[j & 1] : kPairX ? 64 * (q >> 2) + 16 * ((unsigned)lane_here & 3)
+                                                                     : ((unsigned)lane_here >> 4) * 16;
+                x_off[j] = (unsigned)__umul24(min(xr, (unsigned)(M - 1)), rowbytes) + within;
+            }
             if constexpr (XDMA) {
                 static_for<T>([&](auto t) {
-#pragma unroll
-                    for (int u = 0; u < 2; ++u)
-                        dma16<false, t() * kTileRowBytes>(xbase, x_off[f][u],
-                                                          my_lds + ((R + f) * T + t()) * kTileBytes + u * 1024);
+                    dma16_at<false, t() * kTileRowBytes, (R * T + t()) * kTileBytes>(xbase, x_off[0], my_lds + f * T * kTileBytes);
+                    dma16_at<false, t() * kTileRowBytes, (R * T + t()) * kTileBytes + 1024>(xbase, x_off[1],
+                                                                                              my_lds + f * T * kTileBytes);
                 });
             } else if constexpr (kPairX) {
                 static_for<2 * T>([&](auto j) {
-                    load16_untracked<(j() >> 2) * 2 * kTileRowBytes>(xg[XDMA ? 0 : j() >> 1][j() & 1][f], xbase, x_off[f][j() & 3]);
+                    load16_untracked<(j() >> 2) * 2 * kTileRowBytes>(xg[XDMA ? 0 : j() >> 1][j() & 1][f], xbase, x_off[j() & 3]);
                 });
             } else {
                 static_for<2 * T>([&](auto j) {  // tile j / 2, step j % 2
-                    load16_untracked<(j() >> 1) * kTileRowBytes + (j() & 1) * 64>(xg[XDMA ? 0 : j() >> 1][j() & 1][f], xbase, x_off[f][0]);
+                    load16_untracked<(j() >> 1) * kTileRowBytes + (j() & 1) * 64>(xg[XDMA ? 0 : j() >> 1][j() & 1][f], xbase, x_off[0]);
                 });
             }
         }
-        if constexpr (kTilesBeforeX > 0)
-            issue_w(0, kHead, kTail);
-#pragma unroll
-        for (int rg = kGroupsBeforeX + (kTilesBeforeX > 0 ? 1 : 0); rg < R; ++rg)
-            issue_w(rg, kZero, kAllTiles);
+    }
+    if constexpr (T > 1)
+        issue_w(kZero, kOne, kRestOfGroup);
+    static_for<R - 1>([&](auto g) { issue_w(std::integral_constant<int, decltype(g)::value + 1>{}, kZero, kAllTiles); });
     }
 
-    // ---- one row group at a time
-    [&]<int... RG>(std::integer_sequence<int, RG...>) {
-        ([&] {
-            constexpr int rg = RG;
-            [&]<int... TT>(std::integer_sequence<int, TT...>) {
-                ([&] {
-                    constexpr int t = TT;
-                    // Loads younger than tile (rg, t): the rest of this group and the later
-                    // groups.  When X was issued after the first group(s) of W, those groups
-                    // also wait for X, i.e. for everything up to the first group after X.
-                    constexpr int kYounger = ((R - 1 - rg) * T + (T - 1 - t)) * 2;
-                    constexpr int kAfterX = (R - kGroupsBeforeX) * T * 2;
-                    wait_vm_imm<(rg < kGroupsBeforeX && kYounger > kAfterX) ? kAfterX : kYounger>();
-                    if (!XDMA && rg == 0 && t == 0) {
-                        // X has landed: the fragments are formed group by group
-#pragma unroll
-                        for (int f = 0; f < FMX; ++f)
-#pragma unroll
-                            for (int tp = 0; tp < (XDMA ? 1 : T) / (kPairX ? 2 : 1); ++tp) {
-                                constexpr int kTilesHere = kPairX ? 2 : 1;
-#pragma unroll
-                                for (int h = 0; h < 2 * kTilesHere; ++h)
-                                    settle(xg[kTilesHere * tp + (h >> 1)][h & 1][f]);
-                                if constexpr (kPairX)
-                                    quad_transpose(xg[XDMA ? 0 : 2 * tp][0][f], xg[XDMA ? 0 : 2 * tp][1][f],
-                                                   xg[XDMA ? 0 : 2 * tp + 1][0][f], xg[XDMA ? 0 : 2 * tp + 1][1][f], lane);
-                            }
-                    }
-                    // In the paired form a pair of tiles is multiplied when its second tile
-                    // has landed: step s of tile t is register j = 2 * (t % 2) + s of the pair,
-                    // whose chunk 4 * fg + j lies in tile fg / 2 of the pair.
-                    if (kPairX && t % 2 == 0)
-                        return;
-#pragma unroll
-                    for (int tq = (kPairX ? t - 1 : t); tq <= t; ++tq)
-#pragma unroll
-                        for (int s = 0; s < 2; ++s) {
-                            // Tiles before `skip` are not this wave's.  In the paired form every
-                            // register spans both tiles of the pair (lanes with fg < 2 hold the
-                            // first one): the pair is left out if its second tile is, and only
-                            // the first tile's lanes are blanked if just that one is.
-                            if (RAGGED && (kPairX ? t : tq) < skip)
-                                continue;
-                            const bool blank_first = RAGGED && kPairX && t - 1 < skip;
-                            const int j = 2 * (tq & 1) + s;
-                            const int frag = fr * kTileRowBytes + (((4 * s + fg) ^ sw) * 16);
-                            const int off = kPairX ? (rg * T + (t - 1) + (fg >> 1)) * kTileBytes + fr * kTileRowBytes +
-                                                         (((4 * (fg & 1) + j) ^ sw) * 16)
-                                                   : (rg * T + t) * kTileBytes + frag;
-                            v4i w = *(const v4i *)(mine + off);
-                            if (blank_first && fg < 2)
-                                w = (v4i){0, 0, 0, 0};
-                            const v4i wlo = (w << 4) & himask;
-                            const v4i whi = w & himask;
-#pragma unroll
-                            for (int f = 0; f < FMX; ++f) {
-                                const v4i x = XDMA ? *(const v4i *)(mine + ((R + f) * T + t) * kTileBytes + frag)
-                                                   : xg[XDMA ? 0 : tq][s][f];
-                                acc[rg][f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo, (x << 4) & himask, acc[rg][f], 0, 0, 0);
-                                acc[rg][f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi, x & himask, acc[rg][f], 0, 0, 0);
-                            }
-                        }
-                }(), ...);
-            }(std::make_integer_sequence<int, T>{});
+    // Waits until tile t of row group rg has landed: loads complete in issue order, so that
+    // is a wait for a fixed number of younger loads (the rest of this group and the later
+    // groups), which s_waitcnt takes as a constant: hence the switch.  X sits right behind
+    // the first tile of W, so that tile's wait covers X too.  (A store of this wave that is
+    // still on its way counts like a load: the wait then lasts one load longer than needed.)
+    auto wait_tile = [&](int rg, auto tc) {
+        constexpr int kRest = (T - 1 - decltype(tc)::value) * 2;  // of the tile's own group
+        switch (rg) {
+        case 0:
+            wait_vm_imm<(R - 1) * T * 2 + kRest>();
+            break;
+        case 1:
+            wait_vm_imm<(R > 2 ? (R - 2) * T * 2 : 0) + kRest>();
+            break;
+        case 2:
+            wait_vm_imm<(R > 3 ? (R - 3) * T * 2 : 0) + kRest>();
+            break;
+        default:
+            wait_vm_imm<kRest>();
+            break;
+        }
+    };
 
-            // After the last pass the wave's partial sums of this group go where its own
-            // tiles of the group were (nobody else touches that area), while the later
-            // groups are still landing.
-            if (pass == passes - 1) {
-                // Lane (fr, fg) holds Y[m = fr][n = 4 * fg ..+4) of the block; it goes to slot
-                // 16 * fg + (fr ^ 2 * fg), so that the reducing lane 4 * m + j can fetch
-                // (fr = m, fg = j) (neighbouring lanes then store neighbouring 16 bytes of
-                // a row of Y) and neither side runs into LDS bank conflicts.
-                v4i *part = (v4i *)(mine + (rg * T) * kTileBytes) + 16 * fg + (fr ^ (2 * fg));
+    if constexpr (!XDMA) {
+        // X has landed when the first tile of W has: the fragments are formed
+        wait_tile(0, std::integral_constant<int, 0>{});
 #pragma unroll
-                for (int f = 0; f < FMX; ++f)
-                    part[f * 64] = acc[rg][f];
+        for (int f = 0; f < FMX; ++f)
+#pragma unroll
+            for (int tp = 0; tp < (XDMA ? 1 : T) / (kPairX ? 2 : 1); ++tp) {
+                constexpr int kTilesHere = kPairX ? 2 : 1;
+#pragma unroll
+                for (int h = 0; h < 2 * kTilesHere; ++h)
+                    settle(xg[kTilesHere * tp + (h >> 1)][h & 1][f]);
+                if constexpr (kPairX)
+                    quad_transpose(xg[XDMA ? 0 : 2 * tp][0][f], xg[XDMA ? 0 : 2 * tp][1][f],
+                                   xg[XDMA ? 0 : 2 * tp + 1][0][f], xg[XDMA ? 0 : 2 * tp + 1][1][f], lane);
             }
-        }(), ...);
-    }(std::make_integer_sequence<int, R>{});
+    }
+
+    // ---- one row group at a time, in a loop (not unrolled): every group after the first runs
+    //      code that is already in the instruction cache, which matters for the last one --
+    //      nothing overlaps it.
+#pragma unroll 1
+    for (int rg = 0; rg < R; ++rg) {
+        v4i acc[FMX];
+#pragma unroll
+        for (int f = 0; f < FMX; ++f)
+            acc[f] = (v4i){0, 0, 0, 0};
+        const uint8_t *group = mine + rg * T * kTileBytes;
+        static_for<T>([&](auto tc) {
+            constexpr int t = decltype(tc)::value;
+            wait_tile(rg, tc);
+            // In the paired form a pair of tiles is multiplied when its second tile has
+            // landed: step s of tile t is register j = 2 * (t % 2) + s of the pair, whose
+            // chunk 4 * fg + j lies in tile fg / 2 of the pair.
+            if constexpr (!(kPairX && t % 2 == 0)) {
+#pragma unroll
+                for (int tq = (kPairX ? t - 1 : t); tq <= t; ++tq)
+#pragma unroll
+                    for (int s = 0; s < 2; ++s) {
+                        // Tiles before `skip` are not this wave's.  In the paired form every
+                        // register spans both tiles of the pair (lanes with fg < 2 hold the
+                        // first one): the pair is left out if its second tile is, and only
+                        // the first tile's lanes are blanked if just that one is.
+                        if (RAGGED && (kPairX ? t : tq) < skip)
+                            continue;
+                        const bool blank_first = RAGGED && kPairX && t - 1 < skip;
+                        const int j = 2 * (tq & 1) + s;
+                        const int frag = fr * kTileRowBytes + (((4 * s + fg) ^ sw) * 16);
+                        const int off = kPairX ? ((t - 1) + (fg >> 1)) * kTileBytes + fr * kTileRowBytes +
+                                                     (((4 * (fg & 1) + j) ^ sw) * 16)
+                                               : t * kTileBytes + frag;
+                        v4i w = *(const v4i *)(group + off);
+                        if (blank_first && fg < 2)
+                            w = (v4i){0, 0, 0, 0};
+                        const v4i wlo = (w << 4) & himask;
+                        const v4i whi = w & himask;
+#pragma unroll
+                        for (int f = 0; f < FMX; ++f) {
+                            const v4i x = XDMA ? *(const v4i *)(mine + ((R + f) * T + t) * kTileBytes + frag)
+                                               : xg[XDMA ? 0 : tq][s][f];
+                            acc[f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo, (x << 4) & himask, acc[f], 0, 0, 0);
+                            acc[f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi, x & himask, acc[f], 0, 0, 0);
+                        }
+                    }
+            }
+        });
+
+        // Lane (fr, fg) holds Y[m = fr][n = 4 * fg ..+4) of each of the group's FMX blocks; its
+        // element q is added to word 64 * q + lane of the block in LDS, so neither these
+        // additions nor the reads of the storing wave meet a bank conflict.
+        int *const block = sums + rg * FMX * 256 + lane;
+#pragma unroll
+        for (int f = 0; f < FMX; ++f)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                __hip_atomic_fetch_add(block + f * 256 + q * 64, acc[f][q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        asm volatile("" ::: "memory");  // (the compiler keeps the order too)
+        // Then the wave counts itself in: ds_append adds the number of active lanes (64) to the
+        // counter, whose address is the instruction's constant (byte 4 * rg of the workgroup's
+        // LDS), and returns what was there.  A wave's LDS operations take effect in the order
+        // issued, so the wave that finds the counter complete finds all the sums complete.
+        int seen;
+        switch (rg) {
+        case 0:
+            asm volatile("s_mov_b32 m0, 0\n\tds_append %0 offset:0\n\ts_waitcnt lgkmcnt(0)" : "=v"(seen) : : "memory");
+            break;
+        case 1:
+            asm volatile("s_mov_b32 m0, 0\n\tds_append %0 offset:4\n\ts_waitcnt lgkmcnt(0)" : "=v"(seen) : : "memory");
+            break;
+        case 2:
+            asm volatile("s_mov_b32 m0, 0\n\tds_append %0 offset:8\n\ts_waitcnt lgkmcnt(0)" : "=v"(seen) : : "memory");
+            break;
+        default:
+            asm volatile("s_mov_b32 m0, 0\n\tds_append %0 offset:12\n\ts_waitcnt lgkmcnt(0)" : "=v"(seen) : : "memory");
+            break;
+        }
+        // The last wave to arrive at a group stores it, once it is through with its own groups.
+        if (__builtin_amdgcn_readfirstlane(seen) == 64 * (waves * passes - 1))
+            to_store |= 1u << rg;
+    }
     }  // passes
 
-    // ---- the workgroup meets once; one wave per 16 x 16 block adds the S partials up
-    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's partials are in LDS
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
+    if (to_store == 0)
+        return;
+    // (the epilogue's operands are first looked at here, not ahead of the loads)
+    Epilogue ep = ep_all;
+    asm volatile("" : "+s"(ep.bias), "+s"(ep.row_scale), "+s"(ep.col_scale), "+s"(ep.f32));
+    const bool plain = !ep.bias && !ep.row_scale && !ep.col_scale && !ep.f32;
+    const bool whole = (N & 3) == 0 && (rows_here & 3) == 0;
+    const int om = lane >> 2, oj = lane & 3;  // this lane stores Y[om][4 * oj ..+4) of each block
 #pragma unroll 1
-    for (int b = wave; b < R * FMX; b += waves) {
-        const int rg = b / FMX, f = b % FMX;
-        const int om = lane >> 2, oj = lane & 3;  // this lane adds up and stores Y[om][4 * oj ..+4) of the block
-        const v4i *p = (const v4i *)(lds + (rg * T) * kTileBytes) + f * 64 + 16 * oj + (om ^ (2 * oj));
-        // All reads are issued back to back (a loop over the runtime wave count would wait
-        // for each one), eight or sixteen of them; waves that do not exist re-read partial 0
-        // and add zero.
-        auto add_up = [&](auto count) {
-            constexpr int kCount = decltype(count)::value;
-            v4i part[kCount];
+    for (int rg = 0; rg < R; ++rg) {
+        if (!((to_store >> rg) & 1u))
+            continue;
 #pragma unroll
-            for (int wv = 0; wv < kCount; ++wv)
-                part[wv] = p[(size_t)(wv < waves ? wv : 0) * (kWaveTiles * kTileBytes / 16)];
-            v4i total = part[0];
+        for (int f = 0; f < FMX; ++f) {
+            const int *mine_of = sums + (rg * FMX + f) * 256 + 16 * oj + om;
+            v4i sum = {mine_of[0], mine_of[64], mine_of[128], mine_of[192]};
+            sum = sum >> 8;  // both operands carried a factor 16
+            const int m = f * 16 + om;
+            const int nb = rg * 16 + 4 * oj;  // within the workgroup's rows
+            int32_t *dst = Y + (size_t)m * N + n0 + nb;
+            if (plain && whole) {
+                // nothing to load or to convert, and a lane's four outputs exist together or
+                // not at all: this is the path that ends the kernel, a dozen instructions
+                if (m < M && nb < rows_here)
+                    *(v4i *)dst = sum;
+            } else if (m < M) {
+                const float rs = ep.row_scale ? ep.row_scale[m] : 1.f;
 #pragma unroll
-            for (int wv = 1; wv < kCount; ++wv)
-                total += wv < waves ? part[wv] : (v4i){0, 0, 0, 0};
-            return total;
-        };
-        v4i sum = waves <= 8 ? add_up(std::integral_constant<int, 8>{}) : add_up(std::integral_constant<int, 16>{});
-        sum = sum >> 8;  // both operands carried a factor 16
-        const int m = f * 16 + om;
-        const int n = n0 + rg * 16 + 4 * oj;
-        if (m < M) {
-            const float rs = ep.row_scale ? ep.row_scale[m] : 1.f;
+                for (int q = 0; q < 4; ++q) {
+                    const int nn = n0 + (nb + q < rows_here ? nb + q : rows_here - 1);
+                    sum[q] = epilogue_value(ep, sum[q], ep.bias ? ep.bias[nn] : 0, rs,
+                                            ep.col_scale ? ep.col_scale[nn] : 1.f);
+                }
+                if (nb + 3 < rows_here && (N & 3) == 0) {
+                    *(v4i *)dst = sum;
+                } else {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int nn = n + q < n_end ? n + q : n_end - 1;
-                sum[q] = epilogue_value(ep, sum[q], ep.bias ? ep.bias[nn] : 0, rs,
-                                        ep.col_scale ? ep.col_scale[nn] : 1.f);
-            }
-            int32_t *dst = Y + (size_t)m * N + n;
-            if (n + 3 < n_end && (N & 3) == 0) {
-                *(v4i *)dst = sum;
-            } else {
-#pragma unroll
-                for (int q = 0; q < 4; ++q)
-                    if (n + q < n_end)
-                        dst[q] = sum[q];
+                    for (int q = 0; q < 4; ++q)
+                        if (nb + q < rows_here)
+                            dst[q] = sum[q];
+                }
             }
         }
     }
-    // the partial sums have been read: the next run may refill the tiles
-    if (m_first + 16 * FMX < M_all)
-        __builtin_amdgcn_s_barrier();
-    }  // runs of rows of X
 }
 
 // ---- long-W form: many 16-row groups of W per CU, FMX 16-row groups of X.
@@ -736,10 +815,9 @@ struct Plan {
     int lds = 0;
 };
 
-// Which (T, R, FMX, XDMA) combinations exist as kernels.  The partial sums of a row group
-// (FMX KiB per wave) go where the wave's own tiles of that group were (T * 2 KiB), except
-// that with a single row group and X in LDS they may run on into the X tiles; the
-// register-X variant holds 2 * T * FMX 16-byte fragments per lane.
+// Which (T, R, FMX, XDMA) combinations exist as kernels: the register-X variant holds
+// 2 * T * FMX 16-byte fragments per lane, which bounds T * FMX; the other bounds keep the
+// number of instantiations down (shapes outside them have a plan with another T or R).
 constexpr bool variant_exists(int t, int r, int fmx, bool xdma)
 {
     if (xdma)
@@ -759,7 +837,7 @@ bool fit(int tiles, int fmx, int r, bool ragged, Plan &p)
             if (s > 16 || t > tiles || (!ragged && s * t * passes != tiles))
                 continue;
             for (int xd = 1; xd >= 0; --xd) {
-                const int lds = s * t * (r + (xd ? fmx : 0)) * kTileBytes;
+                const int lds = head_bytes(r, fmx) + s * t * (r + (xd ? fmx : 0)) * kTileBytes;
                 if (variant_exists(t, r, fmx, xd != 0) && lds <= kMaxLds &&
                     s * 64 <= max_threads(t, r, fmx, xd != 0)) {
                     p.t = t;
@@ -822,9 +900,20 @@ hipError_t launch_plan(const Plan &p, const void *a, const void *b, void *c, int
     if (p.s == 0)  // set-up call: raise the dynamic-LDS limit of this instantiation
         return hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
     const unsigned grid = (unsigned)((n + p.rows_blk - 1) / p.rows_blk);
-    kern<<<grid, p.s * 64, p.lds, stream>>>((const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k,
-                                            p.rows_blk, p.passes, ep);
-    return hipGetLastError();
+    // More than 16 * FMX rows of X go out in runs of that many, one launch each (the rows of
+    // W are then streamed again, through the caches they were just pulled through).
+    for (int m0 = 0; m0 < m; m0 += 16 * FMX) {
+        Epilogue run_ep = ep;
+        if (run_ep.row_scale)
+            run_ep.row_scale += m0;
+        kern<<<grid, p.s * 64, p.lds, stream>>>((const uint8_t *)a + (size_t)m0 * (size_t)(k >> 1), (const uint8_t *)b,
+                                                (int32_t *)c + (size_t)m0 * (size_t)n, m - m0 < 16 * FMX ? m - m0 : 16 * FMX,
+                                                n, k, p.rows_blk, p.passes, p.s, run_ep);
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess)
+            return e;
+    }
+    return hipSuccess;
     }
 }
 
