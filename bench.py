@@ -56,6 +56,17 @@ def packed_random(torch, rows: int, k: int, seed: int):
     return torch.randint(0, 256, (rows, k // 2), dtype=torch.uint8, device="cuda", generator=g)
 
 
+def packed_normal(torch, rows: int, k: int, seed: int, sigma: float = 2.0):
+    """rows x k/2 bytes of decode-style activations: normal(0, sigma) rounded to nearest and
+    clamped to [-8, 7], packed on the device in the packer's byte layout (element e of a row in
+    byte e/2, even e in the low nibble: utils/packer.cpp:3-18)."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    v = torch.randn((rows, k), device="cuda", generator=g).mul_(sigma).round_().clamp_(-8, 7).to(torch.int16)
+    nib = (v & 0xF).to(torch.uint8)
+    return (nib[:, 0::2] | (nib[:, 1::2] << 4)).contiguous()
+
+
 RAMP_MS = 60.0   # untimed load before the first timed leg, see ramp_clocks
 
 
@@ -145,6 +156,17 @@ def bench_gemm(torch, lib, steps: int, warmup: int):
 
     ramp_clocks(torch, launch, args)
     ev_ms, wall_ms = time_launches(torch, launch, args, steps, warmup)
+    # The reference's own statistic (test/benchmark.cu:93-111): an event pair around every
+    # launch, median over the launches (here without a flush in between: the rotation keeps
+    # the operands cold).
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for i, (e0, e1) in enumerate(pairs):
+        e0.record()
+        launch(args[i % len(args)])
+        e1.record()
+    torch.cuda.synchronize()
+    per_launch = sorted(e0.elapsed_time(e1) for (e0, e1) in pairs)
+    median_ms = per_launch[len(per_launch) // 2]
 
     # The dominant kernel's own duration inside the same sequence of kernels as the timed
     # region: each step converts both operands into caller-owned buffers (what the call above
@@ -175,7 +197,7 @@ def bench_gemm(torch, lib, steps: int, warmup: int):
         if bad != 0:
             raise RuntimeError(f"the caller-owned FP6 entry points failed (status bits {bad})")
         kern_ms = sum(e0.elapsed_time(e1) for (e0, e1) in events[warmup:]) / steps
-    return ev_ms, wall_ms, kernel, kern_ms
+    return ev_ms, wall_ms, kernel, kern_ms, median_ms
 
 
 def bench_decode(torch, lib, steps: int, warmup: int, shapes=None):
@@ -187,7 +209,7 @@ def bench_decode(torch, lib, steps: int, warmup: int, shapes=None):
     for (m, n, k) in (shapes or DECODE_SHAPES):
         wbytes = n * k // 2
         nsets = max(4 if wbytes < (256 << 20) else 2, (768 << 20) // wbytes + 1)   # rotate through > 768 MiB of weights
-        x = packed_random(torch, m, k, 31)
+        x = packed_normal(torch, m, k, 31)   # activations: clamp(round(normal(0, 2))), weights uniform
         sets = [(x, packed_random(torch, n, k, 40 + i), torch.empty((m, n), dtype=torch.int32, device="cuda"))
                 for i in range(nsets)]
         args = [(a.data_ptr(), b.data_ptr(), c.data_ptr(), m, n, k, stream) for (a, b, c) in sets]
@@ -200,6 +222,36 @@ def bench_decode(torch, lib, steps: int, warmup: int, shapes=None):
         del sets
         torch.cuda.empty_cache()
     return out
+
+
+def stream_ceilings(shapes):
+    """Per-launch time of a bare streaming kernel (same read pattern as the decode kernel, no
+    arithmetic, 4*M*N bytes written) for each shape, from tests/host/bin/stream_ceiling: what
+    the device gives a kernel that only streams, launch cost included.  {} when the harness
+    is not built."""
+    import re
+    import subprocess
+
+    exe = ROOT / "tests" / "host" / "bin" / "stream_ceiling"
+    if not exe.exists():
+        return {}
+    try:
+        r = subprocess.run([str(exe)] + [f"{m}x{n}x{k}" for (m, n, k) in shapes], capture_output=True, text=True, timeout=180)
+    except (OSError, subprocess.TimeoutExpired):
+        return {}
+    out = {}
+    for mm in re.finditer(r"\[CEILING\] (\d+)x(\d+)x(\d+) ([\d.]+) us ([\d.]+) GB/s", r.stdout):
+        out[(int(mm.group(1)), int(mm.group(2)), int(mm.group(3)))] = (float(mm.group(4)), float(mm.group(5)))
+    return out
+
+
+def add_ceilings(entries, ceilings):
+    for d in entries:
+        c = ceilings.get(tuple(d["shape"]))
+        if c:
+            d["bare_stream_us_per_launch"] = c[0]
+            d["bare_stream_GB/s"] = c[1]
+            d["frac_of_bare_stream"] = c[0] / d["us_per_launch"]
 
 
 def bench_int8_kernel(torch, lib, steps: int, warmup: int):
@@ -329,7 +381,7 @@ def main() -> int:
         del src, dst
         torch.cuda.empty_cache()
 
-    ev_ms, wall_ms, kernel, kern_ms = bench_gemm(torch, lib, args.steps, args.warmup)
+    ev_ms, wall_ms, kernel, kern_ms, median_ms = bench_gemm(torch, lib, args.steps, args.warmup)
     ops = 2.0 * M * N * K
     tops_kernel = ops / (kern_ms * 1e-3) / 1e12
     tops_wall = ops / (wall_ms * 1e-3) / 1e12
@@ -346,12 +398,17 @@ def main() -> int:
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": wall_ms,
+        "median_ms": median_ms,
+        "median_TOPS": 2.0 * M * N * K / (median_ms * 1e-3) / 1e12,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "fp6" if kernel == "fp6" else "int8",
         "dtype_note": ("s4 operands re-encoded exactly as FP6 E2M3, fp32 accumulation of integers below 2^24: "
-                       "bit-identical to int32 arithmetic") if kernel == "fp6" else "s4 widened to int8, int32 accumulation",
+                       "bit-identical to int32 arithmetic.  pct_of_int8_mfma_peak divides this throughput by the "
+                       "int8 MFMA peak the metric names although the kernel issues FP6 MFMAs (peak 10.1 PFLOP/s): "
+                       "a ratio across units; roofline.frac is the one against the issued instruction's own peak")
+        if kernel == "fp6" else "s4 widened to int8, int32 accumulation",
         "data": "synthetic",
         "config": {"workload": "M=N=K=8192 s4*s4->s32 GEMM, uniform [-8,7], 3 rotating operand sets",
                    "untimed_clock_ramp_ms": RAMP_MS,
@@ -360,6 +417,8 @@ def main() -> int:
         "roofline": {"bound": "mfma", "achieved": tops_kernel, "peak": peak,
                      "unit": "TFLOP/s", "frac": tops_kernel / peak,
                      "traffic": measured_traffic(kernel),
+                     "traffic_source": "static: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs recorded in "
+                                       "profiles/fp6_gemm_8192_and_decode_hbm_traffic.md, not measured by this run",
                      "kernel": kernel_name,
                      "note": "2*M*N*K multiply-adds per launch / mean duration of the GEMM kernel itself: a HIP "
                              "event pair around each of its launches on caller-owned converted operands, in the "
@@ -370,11 +429,19 @@ def main() -> int:
     if not args.no_decode:
         dec = bench_decode(torch, lib, args.steps, args.warmup)
         result["decode"] = dec
-        big = [d for d in dec if d["shape"] != [16, 4096, 4096]]
-        result["decode_GB/s_M16"] = sum(d["GB/s"] for d in big) / len(big)
+        result["decode_GB/s_M16"] = sum(d["GB/s"] for d in dec) / len(dec)
+        result["decode_GB/s_M16_min"] = min(d["GB/s"] for d in dec)
+        result["decode_M16_shapes"] = [d["shape"] for d in dec]
+        result["decode_note"] = ("mean time per launch of back-to-back launches over rotating weights (> 768 MiB); "
+                                 "bare_stream_*: a kernel that only streams the same bytes in the same pattern, "
+                                 "launched the same way (tests/host/stream_ceiling.cpp)")
         result["decode_other_M"] = bench_decode(torch, lib, args.steps, args.warmup, DECODE_OTHER_M)
         if not args.no_extra:
             result["decode_large_W"] = bench_decode(torch, lib, args.steps, args.warmup, DECODE_LARGE_W)
+        torch.cuda.synchronize()
+        all_dec = result["decode"] + result["decode_other_M"] + result.get("decode_large_W", [])
+        ceilings = stream_ceilings([tuple(d["shape"]) for d in all_dec])
+        add_ceilings(all_dec, ceilings)
     if not args.no_extra:
         result["int8_kernel"] = bench_int8_kernel(torch, lib, max(10, args.steps // 2), args.warmup)
         result["vendor"] = vendor_line()

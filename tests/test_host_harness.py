@@ -20,7 +20,7 @@ def _binary(name: str) -> Path:
 
 
 def test_harness_binaries_link_against_the_library():
-    for name in ("correctness", "benchmark", "vendor_compare"):
+    for name in ("correctness", "benchmark", "vendor_compare"):  # (stream_ceiling does not use the library)
         out = subprocess.run(["ldd", str(_binary(name))], check=True, capture_output=True, text=True).stdout
         assert "libint4linear.so" in out and "not found" not in out, out
 
@@ -79,3 +79,19 @@ def test_vendor_comparison_agrees_bit_for_bit(gpu):
     assert len(lines) == 4, r.stdout
     for l in lines:
         assert "results identical" in l or "offers no int8" in l, l
+
+
+def test_stream_ceiling_usage_error_without_a_device():
+    r = subprocess.run([str(_binary("stream_ceiling"))], capture_output=True, text=True)
+    assert r.returncode == 2 and "usage" in r.stderr
+    r = subprocess.run([str(_binary("stream_ceiling")), "16x4096x100"], capture_output=True, text=True)
+    assert r.returncode == 2
+
+
+@pytest.mark.gpu
+def test_stream_ceiling_reports_a_rate(gpu):
+    r = subprocess.run([str(_binary("stream_ceiling")), "--steps", "50", "16x4096x4096", "16x14336x4096"],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout + r.stderr
+    rates = re.findall(r"\[CEILING\] \d+x\d+x\d+ ([\d.]+) us ([\d.]+) GB/s", r.stdout)
+    assert len(rates) == 2 and all(0.5 < float(us) < 100 and float(gbs) > 100 for us, gbs in rates), r.stdout
