@@ -95,3 +95,16 @@ def test_stream_ceiling_reports_a_rate(gpu):
     assert r.returncode == 0, r.stdout + r.stderr
     rates = re.findall(r"\[CEILING\] \d+x\d+x\d+ ([\d.]+) us ([\d.]+) GB/s", r.stdout)
     assert len(rates) == 2 and all(0.5 < float(us) < 100 and float(gbs) > 100 for us, gbs in rates), r.stdout
+
+
+def test_mfma_ceiling_usage_error_without_a_device():
+    r = subprocess.run([str(_binary("mfma_ceiling")), "--bogus"], capture_output=True, text=True)
+    assert r.returncode == 2 and "usage" in r.stderr
+
+
+@pytest.mark.gpu
+def test_mfma_ceiling_reports_rates(gpu):
+    r = subprocess.run([str(_binary("mfma_ceiling")), "--iters", "500"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout + r.stderr
+    rows = re.findall(r"\[MFMA\] (int8|fp6) .*? ([\d.]+) TOPS +([\d.]+) GHz", r.stdout)
+    assert len(rows) == 8 and all(float(t) > 500 and 0.5 < float(g) < 3.0 for _, t, g in rows), r.stdout
