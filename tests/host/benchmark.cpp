@@ -3,7 +3,13 @@
 // by its own event pair, median reported as 2*M*N*K / t in TOPS ("[PERF] ... TOPS").
 //
 //   benchmark [--kernel auto|simple|mfma|mfma128|mfma256|skinny|fp6] [--epilogue none|bias|f32]
-//             [--iters I] [--warmup W] [--no-flush] MxNxK ...
+//             [--entry v0|v1|v2|v10|v11|v20|v21] [--iters I] [--warmup W] [--no-flush] MxNxK ...
+//
+// --entry times one of the reference's blocking linear_vN_launch entry points instead (each a
+// step of this library's kernel history, kernels/linear_v0.h:168 ... linear_v21.h:760): wall
+// time of the call between two device synchronisations, which is what the reference's own
+// callers see (kernels/linear_v21.cu:37-39), and under rocprofv3 --kernel-trace the kernels of
+// that step.
 //
 // --epilogue bias times int4linear_linear_s32 (bias add fused into the store), f32 times
 // int4linear_linear_f32 (bias, per-row and per-column scales, float output).
@@ -34,7 +40,7 @@ int kernel_id(const std::string &name)
 
 int main(int argc, char **argv)
 {
-    std::string kernel = "auto", epilogue = "none";
+    std::string kernel = "auto", epilogue = "none", entry;
     int iters = 50, warmup = 5;
     bool flush = true;
     std::vector<Shape> shapes;
@@ -43,6 +49,7 @@ int main(int argc, char **argv)
         Shape s;
         if (a == "--kernel" && i + 1 < argc) kernel = argv[++i];
         else if (a == "--epilogue" && i + 1 < argc) epilogue = argv[++i];
+        else if (a == "--entry" && i + 1 < argc) entry = argv[++i];
         else if (a == "--iters" && i + 1 < argc) iters = std::atoi(argv[++i]);
         else if (a == "--warmup" && i + 1 < argc) warmup = std::atoi(argv[++i]);
         else if (a == "--no-flush") flush = false;
@@ -50,6 +57,21 @@ int main(int argc, char **argv)
         else {
             std::fprintf(stderr, "usage: %s [--kernel auto|simple|mfma|mfma128|mfma256|skinny|fp6] [--iters I] [--warmup W] "
                                  "[--no-flush] MxNxK ...\n", argv[0]);
+            return 2;
+        }
+    }
+    using Launcher = void (*)(void *, void *, void *, int, int, int);
+    Launcher entry_fn = nullptr;
+    if (!entry.empty()) {
+        if (entry == "v0") entry_fn = linear_v0_launch;
+        else if (entry == "v1") entry_fn = linear_v1_launch;
+        else if (entry == "v2") entry_fn = linear_v2_launch;
+        else if (entry == "v10") entry_fn = linear_v10_launch;
+        else if (entry == "v11") entry_fn = linear_v11_launch;
+        else if (entry == "v20") entry_fn = linear_v20_launch;
+        else if (entry == "v21") entry_fn = linear_v21_launch;
+        else {
+            std::fprintf(stderr, "bad --entry\n");
             return 2;
         }
     }
@@ -86,6 +108,10 @@ int main(int argc, char **argv)
             HIP_OK(hipMemcpy(cscale.p, c.data(), cscale.bytes, hipMemcpyHostToDevice));
         }
         auto launch = [&]() {
+            if (entry_fn) {
+                entry_fn(xd.p, wd.p, yd.p, m, n, k);  // blocks until the device is done
+                return;
+            }
             int st;
             if (epilogue == "bias")
                 st = int4linear_linear_s32(xd.p, wd.p, (const int *)bias.p, yd.p, m, n, k, kid, nullptr);
@@ -119,7 +145,8 @@ int main(int argc, char **argv)
         const double ops = 2.0 * m * (double)n * k;
         const double bytes = (double)m * k / 2 + (double)n * k / 2 + 4.0 * m * n;
         std::printf("[PERF] %dx%dx%d kernel=%s epilogue=%s median %.4f ms (min %.4f)  %lf TOPS  %.1f GB/s\n", m, n, k,
-                    kid == INT4LINEAR_KERNEL_AUTO ? int4linear_kernel_for_shape(m, n, k) : kernel.c_str(),
+                    entry_fn ? ("linear_" + entry + "_launch").c_str()
+                    : kid == INT4LINEAR_KERNEL_AUTO ? int4linear_kernel_for_shape(m, n, k) : kernel.c_str(),
                     epilogue.c_str(), median_ms, (double)ms[0], ops / (median_ms * 1e9), bytes / (median_ms * 1e6));
     }
     HIP_OK(hipEventDestroy(start));

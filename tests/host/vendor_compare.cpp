@@ -6,7 +6,10 @@
 // bit for bit with this library's, then both are timed with the benchmark harness's
 // protocol (5 warm-ups, 50 iterations, cache-cleaning fill, per-launch events, median).
 //
-//   vendor_compare [--iters I] [--warmup W] MxNxK ...
+//   vendor_compare [--iters I] [--warmup W] [--readme-sweep] MxNxK ...
+//
+// --readme-sweep adds the two shape families of the reference README's chart (README.md:57-62:
+// M = N = K and 2M = 2N = K, 1024 ... 8192) and prints the results once more as one table.
 #include <hipblaslt/hipblaslt.h>
 
 #include "harness_common.h"
@@ -70,15 +73,22 @@ double median_ms(F &&launch, int warmup, int iters, void *fill, size_t fill_byte
 int main(int argc, char **argv)
 {
     int iters = 50, warmup = 5;
+    bool table = false;
     std::vector<Shape> shapes;
     for (int i = 1; i < argc; ++i) {
         const std::string a = argv[i];
         Shape s;
         if (a == "--iters" && i + 1 < argc) iters = std::atoi(argv[++i]);
         else if (a == "--warmup" && i + 1 < argc) warmup = std::atoi(argv[++i]);
-        else if (parse_shape(argv[i], s)) shapes.push_back(s);
+        else if (a == "--readme-sweep") {
+            // The two families of the reference README's chart (README.md:57-62): M = N = K and
+            // 2M = 2N = K, custom kernel against the vendor library, as one table.
+            table = true;
+            for (int d : {1024, 2048, 4096, 8192}) shapes.push_back({d, d, d});
+            for (int d : {1024, 2048, 4096, 8192}) shapes.push_back({d, d, 2 * d});
+        } else if (parse_shape(argv[i], s)) shapes.push_back(s);
         else {
-            std::fprintf(stderr, "usage: %s [--iters I] [--warmup W] MxNxK ...\n", argv[0]);
+            std::fprintf(stderr, "usage: %s [--iters I] [--warmup W] [--readme-sweep] MxNxK ...\n", argv[0]);
             return 2;
         }
     }
@@ -91,6 +101,7 @@ int main(int argc, char **argv)
     const size_t fill_bytes = 512ull << 20, ws_bytes = 128ull << 20;
     DeviceBuffer fill(fill_bytes), workspace(ws_bytes), mismatches(sizeof(unsigned long long));
     bool all_equal = true;
+    std::vector<std::string> rows;
 
     for (const Shape &s : shapes) {
         const int m = s.m, n = s.n, k = s.k;
@@ -159,6 +170,11 @@ int main(int argc, char **argv)
                         "ratio %.2fx | results %s\n",
                         m, n, k, t_vendor, ops / (t_vendor * 1e9), int4linear_kernel_for_shape(m, n, k), t_ours,
                         ops / (t_ours * 1e9), t_vendor / t_ours, bad == 0 ? "identical" : "DIFFER");
+            char row[256];
+            std::snprintf(row, sizeof(row), "| %d x %d x %d | %s | %.1f | %.0f | %.1f | %.0f | %.2fx | %s |", m, n, k,
+                          int4linear_kernel_for_shape(m, n, k), t_ours * 1e3, ops / (t_ours * 1e9), t_vendor * 1e3,
+                          ops / (t_vendor * 1e9), t_vendor / t_ours, bad == 0 ? "identical" : "DIFFER");
+            rows.push_back(row);
         }
         BLT_OK(hipblasLtMatmulPreferenceDestroy(pref));
         BLT_OK(hipblasLtMatrixLayoutDestroy(lw));
@@ -167,5 +183,11 @@ int main(int argc, char **argv)
         BLT_OK(hipblasLtMatmulDescDestroy(desc));
     }
     BLT_OK(hipblasLtDestroy(handle));
+    if (table) {
+        std::printf("\n| M x N x K | kernel | int4linear us | TOPS | hipBLASLt int8 us | TOPS | ratio | results |\n"
+                    "|---|---|---|---|---|---|---|---|\n");
+        for (const std::string &r : rows)
+            std::printf("%s\n", r.c_str());
+    }
     return all_equal ? 0 : 1;
 }
