@@ -185,9 +185,14 @@ constexpr int head_bytes(int r, int fmx) { return 1024 + r * fmx * 1024; }
 // only the last group's share is exposed after the last byte arrives.
 template <int T, int R, int FMX, bool XDMA, bool RAGGED>
 __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(const uint8_t *X, const uint8_t *W, int32_t *Y,
-                                                                              int M, int N, int K, int rows_blk, int passes,
-                                                                              int waves, Epilogue ep_all)
+                                                                              v4i dims, Epilogue ep_all)
 {
+    // dims: { M | passes << 8 | S << 16, N, K, rows_blk } -- one argument instead of six: the
+    // host's cost of a launch grows with the number of arguments (0.1 us each), and these
+    // launches are short enough for that to show.
+    int M = dims[0] & 0xFF, passes = (dims[0] >> 8) & 0xFF;
+    const int waves = dims[0] >> 16;
+    const int N = dims[1], K = dims[2], rows_blk = dims[3];
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int kWaveTiles = T * (R + (XDMA ? FMX : 0));
     constexpr int kHead = head_bytes(R, FMX);
@@ -906,9 +911,10 @@ hipError_t launch_plan(const Plan &p, const void *a, const void *b, void *c, int
         Epilogue run_ep = ep;
         if (run_ep.row_scale)
             run_ep.row_scale += m0;
+        const int rows = m - m0 < 16 * FMX ? m - m0 : 16 * FMX;
         kern<<<grid, p.s * 64, p.lds, stream>>>((const uint8_t *)a + (size_t)m0 * (size_t)(k >> 1), (const uint8_t *)b,
-                                                (int32_t *)c + (size_t)m0 * (size_t)n, m - m0 < 16 * FMX ? m - m0 : 16 * FMX,
-                                                n, k, p.rows_blk, p.passes, p.s, run_ep);
+                                                (int32_t *)c + (size_t)m0 * (size_t)n,
+                                                (v4i){rows | (p.passes << 8) | (p.s << 16), n, k, p.rows_blk}, run_ep);
         const hipError_t e = hipGetLastError();
         if (e != hipSuccess)
             return e;
@@ -1099,16 +1105,37 @@ bool skinny_preferred(int m, int n, int k, const DeviceInfo &)
     return m <= 64 && skinny_supports(m, n, k);
 }
 
+namespace {
+
+// The plan of the shape a host thread asked for last: a decode loop calls with a handful of
+// shapes over and over, and next to a kernel of a few microseconds the plan search (some
+// hundred candidate splits) is not free.
+struct PlanCache {
+    int m = -1, n = -1, k = -1, cus = -1;
+    int kind = 0;  // 1: long-W form, 2: tiled form, 3: neither
+    StreamPlan sp;
+    Plan p;
+};
+thread_local PlanCache t_plan;
+
+}  // namespace
+
 hipError_t launch_skinny(const void *a, const void *b, void *c, int m, int n, int k,
                          const Epilogue &ep, const DeviceInfo &dev, hipStream_t stream)
 {
-    StreamPlan sp;
-    if (make_stream_plan(m, n, k, dev.cu_count, sp))
-        return dispatch_stream(sp, a, b, c, m, n, k, ep, stream);
-    Plan p;
-    if (make_plan(m, n, k, dev.cu_count, p))
-        return p.xdma ? dispatch_t<true>(p, a, b, c, m, n, k, ep, stream)
-                      : dispatch_t<false>(p, a, b, c, m, n, k, ep, stream);
+    PlanCache &pc = t_plan;
+    if (pc.m != m || pc.n != n || pc.k != k || pc.cus != dev.cu_count) {
+        pc.kind = make_stream_plan(m, n, k, dev.cu_count, pc.sp) ? 1 : make_plan(m, n, k, dev.cu_count, pc.p) ? 2 : 3;
+        pc.m = m;
+        pc.n = n;
+        pc.k = k;
+        pc.cus = dev.cu_count;
+    }
+    if (pc.kind == 1)
+        return dispatch_stream(pc.sp, a, b, c, m, n, k, ep, stream);
+    if (pc.kind == 2)
+        return pc.p.xdma ? dispatch_t<true>(pc.p, a, b, c, m, n, k, ep, stream)
+                         : dispatch_t<false>(pc.p, a, b, c, m, n, k, ep, stream);
     if (m > 64)
         return hipErrorInvalidConfiguration;  // skinny_supports() says no
     switch ((m + 15) / 16) {
