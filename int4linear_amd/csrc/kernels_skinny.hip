@@ -385,6 +385,26 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
             }
     }
 
+    // With several row groups of W and of X, X is widened once per pass where the registers
+    // allow it (16 per tile and row group of X) instead of once per row group of W.
+    constexpr bool kWideX = R > 1 && FMX > 1 && T * FMX <= 4;
+    v4i xw[kWideX ? T : 1][2][kWideX ? FMX : 1][2];
+    if constexpr (kWideX) {
+        if constexpr (XDMA)
+            wait_tile(0, std::integral_constant<int, 0>{});  // X sits right behind the first tile of W
+#pragma unroll
+        for (int t = 0; t < T; ++t)
+#pragma unroll
+            for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+                for (int f = 0; f < FMX; ++f) {
+                    const int frag = fr * kTileRowBytes + (((4 * s2 + fg) ^ sw) * 16);
+                    const v4i x = XDMA ? *(const v4i *)(mine + ((R + f) * T + t) * kTileBytes + frag) : xg[XDMA ? 0 : t][s2][f];
+                    xw[t][s2][f][0] = (x << 4) & himask;
+                    xw[t][s2][f][1] = x & himask;
+                }
+    }
+
     // ---- one row group at a time, in a loop (not unrolled): every group after the first runs
     //      code that is already in the instruction cache, which matters for the last one --
     //      nothing overlaps it.
@@ -425,10 +445,15 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
                         const v4i whi = w & himask;
 #pragma unroll
                         for (int f = 0; f < FMX; ++f) {
-                            const v4i x = XDMA ? *(const v4i *)(mine + ((R + f) * T + t) * kTileBytes + frag)
-                                               : xg[XDMA ? 0 : tq][s][f];
-                            acc[f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo, (x << 4) & himask, acc[f], 0, 0, 0);
-                            acc[f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi, x & himask, acc[f], 0, 0, 0);
+                            if constexpr (kWideX) {
+                                acc[f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo, xw[tq][s][f][0], acc[f], 0, 0, 0);
+                                acc[f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi, xw[tq][s][f][1], acc[f], 0, 0, 0);
+                            } else {
+                                const v4i x = XDMA ? *(const v4i *)(mine + ((R + f) * T + t) * kTileBytes + frag)
+                                                   : xg[XDMA ? 0 : tq][s][f];
+                                acc[f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo, (x << 4) & himask, acc[f], 0, 0, 0);
+                                acc[f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi, x & himask, acc[f], 0, 0, 0);
+                            }
                         }
                     }
             }
