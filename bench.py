@@ -1,7 +1,8 @@
 #!/usr/bin/env python3
 """Benchmark of the packed-int4 linear-layer GEMM on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-decode] [--no-extra] [--calibrate-copy]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-decode] [--no-extra] [--no-vendor]
+                    [--no-ceiling] [--calibrate-copy]
 
 A step is one GEMM launch C[MxN] = A[MxK] * B[NxK]^T through the library's C ABI
 (int4linear_gemm_s4s4s32, asynchronous, on torch's current stream).  The workload is
@@ -353,7 +354,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="skip the decode-shape leg")
-    ap.add_argument("--no-extra", action="store_true", help="skip the int8-kernel and vendor legs")
+    ap.add_argument("--no-extra", action="store_true", help="skip the int8-kernel, large-W decode and vendor legs")
+    ap.add_argument("--no-vendor", action="store_true", help="skip the vendor-library leg (a child process)")
+    ap.add_argument("--no-ceiling", action="store_true", help="skip the bare-stream ceiling leg (a child process)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run four plain 1 GiB device copies first (a kernel of known traffic "
                          "to scale hardware byte counters by when profiling)")
@@ -441,11 +444,12 @@ def main() -> int:
             result["decode_large_W"] = bench_decode(torch, lib, args.steps, args.warmup, DECODE_LARGE_W)
         torch.cuda.synchronize()
         all_dec = result["decode"] + result["decode_other_M"] + result.get("decode_large_W", [])
-        ceilings = stream_ceilings([tuple(d["shape"]) for d in all_dec])
-        add_ceilings(all_dec, ceilings)
+        if not args.no_ceiling:
+            add_ceilings(all_dec, stream_ceilings([tuple(d["shape"]) for d in all_dec]))
     if not args.no_extra:
         result["int8_kernel"] = bench_int8_kernel(torch, lib, max(10, args.steps // 2), args.warmup)
-        result["vendor"] = vendor_line()
+        if not args.no_vendor:
+            result["vendor"] = vendor_line()
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline()
     print(json.dumps(result))
