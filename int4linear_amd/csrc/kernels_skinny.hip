@@ -187,15 +187,25 @@ template <int T, int R, int FMX, bool XDMA, bool RAGGED>
 __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(const uint8_t *X, const uint8_t *W, int32_t *Y,
                                                                               v4i dims, Epilogue ep_all)
 {
-    // dims: { M | passes << 8 | S << 16, N, K, rows_blk } -- one argument instead of six: the
-    // host's cost of a launch grows with the number of arguments (0.1 us each), and these
-    // launches are short enough for that to show.
+    // dims: { M | passes << 8 | S << 16 | plain << 24, N, K, rows_blk } -- one argument instead
+    // of seven: the host's cost of a launch grows with the number of arguments (0.1 us each),
+    // and these launches are short enough for that to show.  `plain` says that ep_all is all
+    // zero, which the storing wave then knows without loading it.
     int M = dims[0] & 0xFF, passes = (dims[0] >> 8) & 0xFF;
-    const int waves = dims[0] >> 16;
+    const int waves = (dims[0] >> 16) & 0xFF;
+    const bool plain = (dims[0] >> 24) & 1;
     const int N = dims[1], K = dims[2], rows_blk = dims[3];
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int kWaveTiles = T * (R + (XDMA ? FMX : 0));
     constexpr int kHead = head_bytes(R, FMX);
+    // Row groups of W whose loads are in flight ahead of the one being multiplied.  With one
+    // row group of X a wave issues everything at once.  With more, a wave has X (16 * FMX
+    // rows of its K slice) to fetch as well, the CU's queue of outstanding loads fills up, a
+    // wave then sits in the issue of its later loads while its first row groups are waiting
+    // in LDS, and all waves reach the ends of their chains of row groups together and late:
+    // there the later groups are issued one at a time, each when the group before it has been
+    // multiplied (64 x 14336 x 4096: 11.3 -> 10.7 us, with the rotation below 9.9 us).
+    constexpr int kAhead = (FMX >= 2 && R > 1) ? 1 : R - 1;
 
     // ---- first of all, the wave's first two loads (tile 0 of row group 0, first pass).
     //      Nothing overlaps the time before a wave's first load, so these go out after as few
@@ -212,17 +222,24 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
         // Lane p of a direct-to-LDS instruction lands at 16*p: tile row p/8 (+8 for the second
         // instruction of a tile), slot p%8, so it fetches chunk slot ^ swizzle.
         const unsigned lrow = (unsigned)lane >> 3, c8 = (unsigned)lane & 7;
-        const unsigned lim = (unsigned)min(rows_here - 1, 15);
+        const unsigned g0 = 16u * (wave & (R - 1));  // the wave's first row group (see `rot`)
+        const unsigned lim = (unsigned)(rows_here - 1);
         const int skip0 = RAGGED ? max(0, (wave + 1) * T - K / kTileK) : 0;
         const uint8_t *base = W + (size_t)n0 * rowbytes + (size_t)(wave * T - skip0) * kTileRowBytes;
         const unsigned first_lds = lds_base + kHead + wave * kWaveTiles * kTileBytes;
-        dma16_at<true, 0, 0>(base, (unsigned)__umul24(min(lrow, lim), rowbytes) + ((c8 ^ (lrow >> 1)) << 4), first_lds);
-        dma16_at<true, 0, 1024>(base, (unsigned)__umul24(min(lrow + 8, lim), rowbytes) + ((c8 ^ (4 + (lrow >> 1))) << 4),
+        dma16_at<true, 0, 0>(base, (unsigned)__umul24(min(g0 + lrow, lim), rowbytes) + ((c8 ^ (lrow >> 1)) << 4), first_lds);
+        dma16_at<true, 0, 1024>(base, (unsigned)__umul24(min(g0 + lrow + 8, lim), rowbytes) + ((c8 ^ (4 + (lrow >> 1))) << 4),
                                 first_lds);
     }
     asm volatile("" : "+v"(lane), "+s"(wave), "+s"(rowbytes), "+s"(n0), "+s"(rows_here), "+s"(M), "+s"(passes));
 
     const unsigned my_lds = uniform(lds_base + kHead + wave * kWaveTiles * kTileBytes);
+    // Waves take the row groups in different orders: wave w keeps group (i + w) mod R in its
+    // i-th tiles.  The last wave to arrive at a group stores it, and with one order for all
+    // the slowest wave is the last at every group and stores them all, one after the other,
+    // when everybody else has left; rotated, the groups' last arrivals fall to different
+    // waves, which store side by side (16 x 14336 x 4096: 7.5 -> 7.3 us, 64 rows: 10.7 -> 9.9).
+    const int rot = wave & (R - 1);
     const int himask = (int)0xF0F0F0F0u;
     const uint8_t *mine = lds + kHead + wave * kWaveTiles * kTileBytes;
     int *const arrived = (int *)lds;
@@ -276,8 +293,8 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
     for (int rg = 0; rg < R; ++rg)
 #pragma unroll
         for (int u = 0; u < 2; ++u)
-            w_off[rg][u] = (unsigned)__umul24(min(16 * rg + lrow + 8 * u, (unsigned)(rows_here - 1)), rowbytes) + chunk[u];
-    auto issue_w = [&](auto rgc, auto first, auto count) {  // tiles first .. first + count - 1 of group rg
+            w_off[rg][u] = (unsigned)__umul24(min(16 * ((rg + rot) & (R - 1)) + lrow + 8 * u, (unsigned)(rows_here - 1)), rowbytes) + chunk[u];
+    auto issue_w = [&](auto rgc, auto first, auto count) {  // tiles first .. first + count - 1 of the rg-th group
         constexpr int rg = decltype(rgc)::value;
         static_for<count()>([&](auto i) {
             constexpr int t = first() + i();
@@ -342,30 +359,49 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
     }
     if constexpr (T > 1)
         issue_w(kZero, kOne, kRestOfGroup);
-    static_for<R - 1>([&](auto g) { issue_w(std::integral_constant<int, decltype(g)::value + 1>{}, kZero, kAllTiles); });
+    static_for<kAhead>([&](auto g) { issue_w(std::integral_constant<int, decltype(g)::value + 1>{}, kZero, kAllTiles); });
     }
 
-    // Waits until tile t of row group rg has landed: loads complete in issue order, so that
-    // is a wait for a fixed number of younger loads (the rest of this group and the later
-    // groups), which s_waitcnt takes as a constant: hence the switch.  X sits right behind
-    // the first tile of W, so that tile's wait covers X too.  (A store of this wave that is
-    // still on its way counts like a load: the wait then lasts one load longer than needed.)
-    auto wait_tile = [&](int rg, auto tc) {
+    // Waits until tile t of the wave's i-th row group has landed: loads complete in issue
+    // order, so that is a wait for a fixed number of younger loads (the rest of this group and
+    // the groups issued ahead of it), which s_waitcnt takes as a constant: hence the switch.
+    // X sits right behind the first tile of W, so that tile's wait covers X too.  (A store of
+    // this wave that is still on its way counts like a load: the wait then lasts one load
+    // longer than needed.)
+    auto wait_tile = [&](int i, auto tc) {
         constexpr int kRest = (T - 1 - decltype(tc)::value) * 2;  // of the tile's own group
-        switch (rg) {
-        case 0:
-            wait_vm_imm<(R - 1) * T * 2 + kRest>();
-            break;
-        case 1:
-            wait_vm_imm<(R > 2 ? (R - 2) * T * 2 : 0) + kRest>();
+        switch (min(kAhead, R - 1 - i)) {  // younger groups in flight
+        case 3:
+            wait_vm_imm<(kAhead >= 3 ? 3 : 0) * T * 2 + kRest>();
             break;
         case 2:
-            wait_vm_imm<(R > 3 ? (R - 3) * T * 2 : 0) + kRest>();
+            wait_vm_imm<(kAhead >= 2 ? 2 : 0) * T * 2 + kRest>();
+            break;
+        case 1:
+            wait_vm_imm<(kAhead >= 1 ? 1 : 0) * T * 2 + kRest>();
             break;
         default:
             wait_vm_imm<kRest>();
             break;
         }
+    };
+    // All tiles of the wave's i-th row group, i wave-uniform but not a constant.
+    auto issue_w_dyn = [&](int i) {
+        int lane_here = lane;
+        asm volatile("" : "+v"(lane_here));
+        const unsigned lrow = (unsigned)lane_here >> 3;
+        const unsigned c8 = (unsigned)lane_here & 7;
+        const int first_tile = (pass * waves + wave) * T;
+        const uint8_t *wbase = uniform(W + (size_t)n0 * rowbytes + (size_t)(first_tile - skip) * kTileRowBytes);
+        const unsigned g = 16 * ((i + rot) & (R - 1));
+        const unsigned off0 = (unsigned)__umul24(min(g + lrow, (unsigned)(rows_here - 1)), rowbytes) + ((c8 ^ (lrow >> 1)) << 4);
+        const unsigned off1 = (unsigned)__umul24(min(g + lrow + 8, (unsigned)(rows_here - 1)), rowbytes) +
+                              ((c8 ^ (4 + (lrow >> 1))) << 4);
+        const unsigned grp_lds = uniform(my_lds + i * T * kTileBytes);
+        static_for<T>([&](auto t) {
+            dma16_at<true, t() * kTileRowBytes, t() * kTileBytes>(wbase, off0, grp_lds);
+            dma16_at<true, t() * kTileRowBytes, t() * kTileBytes + 1024>(wbase, off1, grp_lds);
+        });
     };
 
     if constexpr (!XDMA) {
@@ -387,7 +423,7 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
 
     // With several row groups of W and of X, X is widened once per pass where the registers
     // allow it (16 per tile and row group of X) instead of once per row group of W.
-    constexpr bool kWideX = R > 1 && FMX > 1 && T * FMX <= 4;
+    constexpr bool kWideX = R > 1 && FMX > 1 && (T * FMX <= 4 || (max_threads(T, R, FMX, XDMA) == 512 && T * FMX <= 8));
     v4i xw[kWideX ? T : 1][2][kWideX ? FMX : 1][2];
     if constexpr (kWideX) {
         if constexpr (XDMA)
@@ -409,15 +445,19 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
     //      code that is already in the instruction cache, which matters for the last one --
     //      nothing overlaps it.
 #pragma unroll 1
-    for (int rg = 0; rg < R; ++rg) {
+    for (int slot = 0; slot < R; ++slot) {
+        const int rg = (slot + rot) & (R - 1);  // the row group in the wave's slot-th tiles
+        if constexpr (kAhead < R - 1)
+            if (slot >= 1 && slot + kAhead < R)
+                issue_w_dyn(slot + kAhead);
         v4i acc[FMX];
 #pragma unroll
         for (int f = 0; f < FMX; ++f)
             acc[f] = (v4i){0, 0, 0, 0};
-        const uint8_t *group = mine + rg * T * kTileBytes;
+        const uint8_t *group = mine + slot * T * kTileBytes;
         static_for<T>([&](auto tc) {
             constexpr int t = decltype(tc)::value;
-            wait_tile(rg, tc);
+            wait_tile(slot, tc);
             // In the paired form a pair of tiles is multiplied when its second tile has
             // landed: step s of tile t is register j = 2 * (t % 2) + s of the pair, whose
             // chunk 4 * fg + j lies in tile fg / 2 of the pair.
@@ -461,13 +501,16 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
 
         // Lane (fr, fg) holds Y[m = fr][n = 4 * fg ..+4) of each of the group's FMX blocks; its
         // element q is added to word 64 * q + lane of the block in LDS, so neither these
-        // additions nor the reads of the storing wave meet a bank conflict.
+        // additions nor the reads of the storing wave meet a bank conflict.  Both operands
+        // carried a factor 16, so every product, and with it every wave's share, is a multiple
+        // of 256: the shift happens here, where all waves do it side by side, not in the
+        // storing wave.
         int *const block = sums + rg * FMX * 256 + lane;
 #pragma unroll
         for (int f = 0; f < FMX; ++f)
 #pragma unroll
             for (int q = 0; q < 4; ++q)
-                __hip_atomic_fetch_add(block + f * 256 + q * 64, acc[f][q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                __hip_atomic_fetch_add(block + f * 256 + q * 64, acc[f][q] >> 8, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         asm volatile("" ::: "memory");  // (the compiler keeps the order too)
         // Then the wave counts itself in: ds_append adds the number of active lanes (64) to the
         // counter, whose address is the instruction's constant (byte 4 * rg of the workgroup's
@@ -496,12 +539,28 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
 
     if (to_store == 0)
         return;
+    const int om = lane >> 2, oj = lane & 3;  // this lane stores Y[om][4 * oj ..+4) of each block
+    if (plain && ((N | rows_here) & 3) == 0) {
+        // Nothing to load or to convert, and a lane's four outputs exist together or not at
+        // all: the path that ends the kernel in the common case, kept to a few instructions.
+        const int *mine_of = sums + 16 * oj + om;
+        int32_t *dst = Y + (size_t)om * N + n0 + 4 * oj;
+#pragma unroll 1
+        for (int rg = 0; rg < R; ++rg, mine_of += FMX * 256, dst += 16) {
+            if (!((to_store >> rg) & 1u))
+                continue;
+#pragma unroll
+            for (int f = 0; f < FMX; ++f) {
+                const v4i sum = {mine_of[f * 256], mine_of[f * 256 + 64], mine_of[f * 256 + 128], mine_of[f * 256 + 192]};
+                if (f * 16 + om < M && rg * 16 + 4 * oj < rows_here)
+                    *(v4i *)(dst + (size_t)f * 16 * N) = sum;
+            }
+        }
+        return;
+    }
     // (the epilogue's operands are first looked at here, not ahead of the loads)
     Epilogue ep = ep_all;
     asm volatile("" : "+s"(ep.bias), "+s"(ep.row_scale), "+s"(ep.col_scale), "+s"(ep.f32));
-    const bool plain = !ep.bias && !ep.row_scale && !ep.col_scale && !ep.f32;
-    const bool whole = (N & 3) == 0 && (rows_here & 3) == 0;
-    const int om = lane >> 2, oj = lane & 3;  // this lane stores Y[om][4 * oj ..+4) of each block
 #pragma unroll 1
     for (int rg = 0; rg < R; ++rg) {
         if (!((to_store >> rg) & 1u))
@@ -510,16 +569,10 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
         for (int f = 0; f < FMX; ++f) {
             const int *mine_of = sums + (rg * FMX + f) * 256 + 16 * oj + om;
             v4i sum = {mine_of[0], mine_of[64], mine_of[128], mine_of[192]};
-            sum = sum >> 8;  // both operands carried a factor 16
             const int m = f * 16 + om;
             const int nb = rg * 16 + 4 * oj;  // within the workgroup's rows
             int32_t *dst = Y + (size_t)m * N + n0 + nb;
-            if (plain && whole) {
-                // nothing to load or to convert, and a lane's four outputs exist together or
-                // not at all: this is the path that ends the kernel, a dozen instructions
-                if (m < M && nb < rows_here)
-                    *(v4i *)dst = sum;
-            } else if (m < M) {
+            if (m < M) {
                 const float rs = ep.row_scale ? ep.row_scale[m] : 1.f;
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
@@ -930,6 +983,7 @@ hipError_t launch_plan(const Plan &p, const void *a, const void *b, void *c, int
     if (p.s == 0)  // set-up call: raise the dynamic-LDS limit of this instantiation
         return hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
     const unsigned grid = (unsigned)((n + p.rows_blk - 1) / p.rows_blk);
+    const int plain = !ep.bias && !ep.row_scale && !ep.col_scale && !ep.f32;
     // More than 16 * FMX rows of X go out in runs of that many, one launch each (the rows of
     // W are then streamed again, through the caches they were just pulled through).
     for (int m0 = 0; m0 < m; m0 += 16 * FMX) {
@@ -939,7 +993,7 @@ hipError_t launch_plan(const Plan &p, const void *a, const void *b, void *c, int
         const int rows = m - m0 < 16 * FMX ? m - m0 : 16 * FMX;
         kern<<<grid, p.s * 64, p.lds, stream>>>((const uint8_t *)a + (size_t)m0 * (size_t)(k >> 1), (const uint8_t *)b,
                                                 (int32_t *)c + (size_t)m0 * (size_t)n,
-                                                (v4i){rows | (p.passes << 8) | (p.s << 16), n, k, p.rows_blk}, run_ep);
+                                                (v4i){rows | (p.passes << 8) | (p.s << 16) | (plain << 24), n, k, p.rows_blk}, run_ep);
         const hipError_t e = hipGetLastError();
         if (e != hipSuccess)
             return e;
