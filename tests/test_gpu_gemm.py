@@ -108,7 +108,9 @@ def test_cfg4_decode(gpu, host_threads, m, n, k):
     (40, 14336, 6144), (64, 3000, 8192),
     # K covered in several passes
     (64, 4096, 14336), (32, 4100, 14336), (16, 14336, 14336), (64, 500, 20480), (8, 700, 32768), (48, 1000, 12288),
-    # more than 64 rows of X: runs of 64 inside the kernel (only when the kernel is asked for by name)
+    # ... with several row groups of W and of X (later groups issued one ahead, in every pass)
+    (32, 8200, 32768), (64, 8200, 20480), (48, 14336, 12288),
+    # more than 64 rows of X: runs of 64, one launch each (only when the kernel is asked for by name)
     (65, 4096, 4096), (128, 14336, 4096), (100, 3000, 2048), (96, 14336, 512), (128, 600, 14336),
     (200, 520, 1024), (130, 20000, 4096),
     # K whose 128-byte tiles do not split evenly over the waves (43, 17, 74, 19, 23, 61, 5 tiles)
