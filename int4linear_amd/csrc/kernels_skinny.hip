@@ -602,12 +602,16 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
 // it) and the stream never stops between groups.  A step is one tile of one group: wait
 // for it (loads complete in order: NBUF - 2 younger steps stay in flight), read its two
 // fragments, issue the load of step + NBUF - 1 into the tile consumed one step earlier,
-// multiply.  After the last tile of a group the waves leave their partial sums in one of
-// two LDS areas and meet; one wave (they take turns) adds them up and stores the 16 x 16
-// block while the others go on.  That the area of group g is free again at group g + 2
-// follows from the barrier of group g + 1, which its reducer only reaches afterwards.
-// Steps past the last group are issued like the others, as reloads of the last group
+// multiply.  After the last tile of a group a wave adds its share to the group's block of
+// sums in LDS and goes on; the waves meet once per epoch of four groups, and the epoch's
+// blocks are then stored and cleared by as many waves as there are blocks (they take
+// turns) while the others go on.  (One meeting per group, with one wave adding up
+// everybody's partial sums, cost a tenth of the kernel at 128256 rows of W, and more with
+// several row groups of X: 64 x 128256 x 4096 68 -> 60 us.)  Steps past the last group are issued like the others, as reloads of the last group
 // into tiles nobody reads, which keeps the wait counts constant.
+constexpr int kStreamEpoch = 4;  // groups between two meetings of the waves
+constexpr int stream_head_bytes(int fmx) { return 2 * kStreamEpoch * fmx * 1024; }
+
 template <int TW, int NBUF, int FMX>
 __global__ __launch_bounds__(FMX == 1 ? 1024 : 512) void skinny_stream_kernel(const uint8_t *__restrict__ X,
                                                             const uint8_t *__restrict__ W,
@@ -625,13 +629,12 @@ __global__ __launch_bounds__(FMX == 1 ? 1024 : 512) void skinny_stream_kernel(co
     const int g_end = min(groups_total, g_begin + groups_per_block);
     const int fr = lane & 15, fg = lane >> 4, sw = slot_swizzle(fr);
     const int himask = (int)0xF0F0F0F0u;
-    const unsigned ring_lds = (unsigned)(size_t)I4L_LDS(lds) + wave * NBUF * kTileBytes;
-    const uint8_t *ring = lds + wave * NBUF * kTileBytes;
-    // Partial sums: FMX KiB per wave.  With one row group of X there are two such areas, used
-    // by alternate groups of W (one meeting per group); with more there is one (and a second
-    // meeting per group, after the partial sums have been read).
-    constexpr bool kTwoAreas = FMX == 1;
-    uint8_t *parts = lds + waves * NBUF * kTileBytes;
+    // LDS: two sets (for alternate epochs) of one 16 x 16 block of sums per (group of the
+    // epoch, row group of X), then the waves' rings.
+    constexpr int kHead = stream_head_bytes(FMX);
+    const unsigned ring_lds = (unsigned)(size_t)I4L_LDS(lds) + kHead + wave * NBUF * kTileBytes;
+    const uint8_t *ring = lds + kHead + wave * NBUF * kTileBytes;
+    int *const sums = (int *)lds;
 
     // X fragments: packed as loaded and widened at every use, or, where the 256 registers of
     // the eight-wave form have room for it, widened once (several row groups of X make the
@@ -675,12 +678,20 @@ __global__ __launch_bounds__(FMX == 1 ? 1024 : 512) void skinny_stream_kernel(co
         }
     });
 
+    // With the first loads on their way: the sums start at zero, which everybody has to have
+    // seen before anybody adds to them.
+    for (int i = threadIdx.x; i < 2 * kStreamEpoch * FMX * 256; i += waves * 64)
+        sums[i] = 0;
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+
     v4i acc[FMX];
 #pragma unroll
     for (int f = 0; f < FMX; ++f)
         acc[f] = (v4i){0, 0, 0, 0};
     unsigned pos = 0;  // ring position of the current step
-    int reducer = 0;   // first of the FMX waves that add up the current group
+    int turn = 0;      // the wave that takes the first block of the current epoch
 #pragma unroll 1
     for (int g = g_begin; g < g_end; ++g) {
         // (the shift count and mask are hidden from the optimiser in every group: widened
@@ -735,65 +746,66 @@ __global__ __launch_bounds__(FMX == 1 ? 1024 : 512) void skinny_stream_kernel(co
                 }
             }
         });
-        // Partial sums, in the layout that lets the reducing lane 4 * m + j fetch
-        // (fr = m, fg = j) without bank conflicts.
-        v4i *area = (v4i *)(parts + (kTwoAreas ? (g & 1) * waves * 1024 : 0));
+        // The wave adds its share to the group's blocks of sums (every product carries the
+        // factor 256, so the shift happens here; element q of a lane at word 64 * q + lane: no
+        // bank conflicts) and goes on without waiting.  Once per epoch of kStreamEpoch groups
+        // the waves meet; the epoch's blocks are complete then and are stored and cleared by
+        // as many waves as there are blocks, side by side, while the stream goes on.  The next
+        // epoch adds into the other set of blocks, so a set is used again only after the
+        // meeting that follows its clearing.
+        const int e = (g - g_begin) & (kStreamEpoch - 1);
+        const int set = ((g - g_begin) / kStreamEpoch) & 1;
+        int *const epoch_blocks = sums + set * kStreamEpoch * FMX * 256;
+        int *const block = epoch_blocks + e * FMX * 256;
 #pragma unroll
         for (int f = 0; f < FMX; ++f) {
-            area[(wave * FMX + f) * 64 + 16 * fg + (fr ^ (2 * fg))] = acc[f];
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                __hip_atomic_fetch_add(block + f * 256 + q * 64 + lane, acc[f][q] >> 8, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_WORKGROUP);
             acc[f] = (v4i){0, 0, 0, 0};
         }
-        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
-        __builtin_amdgcn_s_barrier();
-        asm volatile("" ::: "memory");
-        // Waves reducer, reducer + 1, ... (mod S) take one 16 x 16 block each.
-        int f_mine = wave - reducer;
-        if (f_mine < 0)
-            f_mine += waves;
-        if (f_mine < FMX) {
-            const int om = lane >> 2, oj = lane & 3;
-            const v4i *p = area + f_mine * 64 + 16 * oj + (om ^ (2 * oj));
-            // four reads in flight at a time (this wave is off the others' critical path, and
-            // its registers hold the X fragments)
-            v4i sum = {0, 0, 0, 0};
-#pragma unroll 1
-            for (int w0 = 0; w0 < waves; w0 += 4) {
-                v4i part[4];
-#pragma unroll
-                for (int q = 0; q < 4; ++q)
-                    part[q] = p[(w0 + q < waves ? w0 + q : 0) * FMX * 64];
-#pragma unroll
-                for (int q = 0; q < 4; ++q)
-                    sum += w0 + q < waves ? part[q] : (v4i){0, 0, 0, 0};
-            }
-            sum = sum >> 8;  // both operands carried a factor 16
-            const int m = 16 * f_mine + om, n = 16 * g + 4 * oj;
-            if (m < M) {
-                const float rs = ep.row_scale ? ep.row_scale[m] : 1.f;
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const int nn = n + q < N ? n + q : N - 1;
-                    sum[q] = epilogue_value(ep, sum[q], ep.bias ? ep.bias[nn] : 0, rs,
-                                            ep.col_scale ? ep.col_scale[nn] : 1.f);
-                }
-                int32_t *dst = Y + (size_t)m * N + n;
-                if (n + 3 < N && (N & 3) == 0) {
-                    *(v4i *)dst = sum;
-                } else {
-#pragma unroll
-                    for (int q = 0; q < 4; ++q)
-                        if (n + q < N)
-                            dst[q] = sum[q];
-                }
-            }
-        }
-        if (!kTwoAreas) {
-            // the partial sums have been read: the area may be written again
-            __builtin_amdgcn_s_waitcnt(0xC07F);
+        if (e == kStreamEpoch - 1 || g + 1 == g_end) {
+            __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
+            const int om = lane >> 2, oj = lane & 3;  // this lane stores Y[om][4 * oj ..+4) of a block
+            // block j of the epoch: group g - e + j / FMX, row group j % FMX of X; the waves take
+            // them in turn, starting with a different wave every epoch
+            int first = wave - turn;
+            if (first < 0)
+                first += waves;
+#pragma unroll 1
+            for (int j = first; j < (e + 1) * FMX; j += waves) {
+                const int f = j % FMX, gj = g - e + j / FMX;
+                int *const mine_of = epoch_blocks + j * 256 + 16 * oj + om;
+                v4i sum = {mine_of[0], mine_of[64], mine_of[128], mine_of[192]};
+                mine_of[0] = 0;
+                mine_of[64] = 0;
+                mine_of[128] = 0;
+                mine_of[192] = 0;
+                const int m = 16 * f + om, n = 16 * gj + 4 * oj;
+                if (m < M) {
+                    const float rs = ep.row_scale ? ep.row_scale[m] : 1.f;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int nn = n + q < N ? n + q : N - 1;
+                        sum[q] = epilogue_value(ep, sum[q], ep.bias ? ep.bias[nn] : 0, rs,
+                                                ep.col_scale ? ep.col_scale[nn] : 1.f);
+                    }
+                    int32_t *dst = Y + (size_t)m * N + n;
+                    if (n + 3 < N && (N & 3) == 0) {
+                        *(v4i *)dst = sum;
+                    } else {
+#pragma unroll
+                        for (int q = 0; q < 4; ++q)
+                            if (n + q < N)
+                                dst[q] = sum[q];
+                    }
+                }
+            }
+            turn = (turn + kStreamEpoch * FMX) % waves;
         }
-        reducer = reducer + FMX >= waves ? reducer + FMX - waves : reducer + FMX;
     }
     wait_vm_imm<0>();  // the reloads past the last group land before the LDS is given up
 }
@@ -1078,7 +1090,7 @@ bool make_stream_plan(int m, int n, int k, int cu_count, StreamPlan &p)
     p.groups_per_block = (groups + cu_count - 1) / cu_count;
     p.grid = (groups + p.groups_per_block - 1) / p.groups_per_block;
     p.bufs = s <= 8 ? 8 : 4;  // up to eight waves: a deeper ring keeps as many bytes in flight
-    p.lds = s * p.bufs * kTileBytes + (fmx == 1 ? 2 : fmx) * s * 1024;
+    p.lds = stream_head_bytes(fmx) + s * p.bufs * kTileBytes;
     return p.lds <= kMaxLds;
 }
 
