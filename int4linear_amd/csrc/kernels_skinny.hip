@@ -607,8 +607,10 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
 // blocks are then stored and cleared by as many waves as there are blocks (they take
 // turns) while the others go on.  (One meeting per group, with one wave adding up
 // everybody's partial sums, cost a tenth of the kernel at 128256 rows of W, and more with
-// several row groups of X: 64 x 128256 x 4096 68 -> 60 us.)  Steps past the last group are issued like the others, as reloads of the last group
-// into tiles nobody reads, which keeps the wait counts constant.
+// several row groups of X: 64 x 128256 x 4096 68 -> 60 us.)  The loads stop with the last
+// tile; the waits of the last NBUF - 2 steps count down accordingly.  (Reloading the last
+// group into tiles nobody reads, which keeps every wait count the same, cost 3 % to 6 %:
+// with seven groups per CU those reloads are a fifth of all loads.)
 constexpr int kStreamEpoch = 4;  // groups between two meetings of the waves
 constexpr int stream_head_bytes(int fmx) { return 2 * kStreamEpoch * fmx * 1024; }
 
@@ -650,8 +652,7 @@ __global__ __launch_bounds__(FMX == 1 ? 1024 : 512) void skinny_stream_kernel(co
 #pragma unroll
     for (int u = 0; u < 2; ++u)
         chunk[u] = ((lane & 7) ^ slot_swizzle(lrow + 8 * u)) * 16;
-    auto issue = [&](int group, auto c, unsigned pos) {
-        const int g = group < g_end ? group : g_end - 1;
+    auto issue = [&](int g, auto c, unsigned pos) {
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             const int row = min(16 * g + lrow + 8 * u, N - 1);
@@ -662,8 +663,10 @@ __global__ __launch_bounds__(FMX == 1 ? 1024 : 512) void skinny_stream_kernel(co
     };
     // The first step of W goes out ahead of X, so that the weight stream starts at once; the
     // first wait of the loop (all but NBUF - 2 steps landed) then covers X as well.
+    int left = (g_end - g_begin) * TW - 1;  // steps after the current one
     static_for<NBUF - 1>([&](auto j) {
-        issue(g_begin + j() / TW, std::integral_constant<int, j() % TW>{}, (unsigned)j());
+        if (j() <= left)
+            issue(g_begin + j() / TW, std::integral_constant<int, j() % TW>{}, (unsigned)j());
         if constexpr (j() == 0) {
             // X: fragment form, once.
             const uint8_t *xbase = X + (size_t)wave * TW * kTileRowBytes;
@@ -699,7 +702,31 @@ __global__ __launch_bounds__(FMX == 1 ? 1024 : 512) void skinny_stream_kernel(co
         int shift = 4, mask = himask;
         asm volatile("" : "+s"(shift), "+s"(mask));
         static_for<TW>([&](auto c) {
-            wait_vm_imm<2 * (NBUF - 2)>();
+            // all but the younger steps in flight have landed: NBUF - 2 of them, fewer at the end
+            if (left >= NBUF - 2) {
+                wait_vm_imm<2 * (NBUF - 2)>();
+            } else {
+                switch (left) {
+                case 0:
+                    wait_vm_imm<0>();
+                    break;
+                case 1:
+                    wait_vm_imm<2>();
+                    break;
+                case 2:
+                    wait_vm_imm<NBUF >= 5 ? 4 : 0>();
+                    break;
+                case 3:
+                    wait_vm_imm<NBUF >= 6 ? 6 : 0>();
+                    break;
+                case 4:
+                    wait_vm_imm<NBUF >= 7 ? 8 : 0>();
+                    break;
+                default:
+                    wait_vm_imm<NBUF >= 8 ? 10 : 0>();
+                    break;
+                }
+            }
             if constexpr (c() == 0) {
                 // (needed once, after the first wait; it costs nothing to say it per group)
 #pragma unroll
@@ -728,7 +755,9 @@ __global__ __launch_bounds__(FMX == 1 ? 1024 : 512) void skinny_stream_kernel(co
             for (int s = 0; s < 2; ++s)
                 w[s] = *(const v4i *)(ring + pos * kTileBytes + fr * kTileRowBytes + (((4 * s + fg) ^ sw) * 16));
             constexpr int ahead = c() + NBUF - 1;
-            issue(g + ahead / TW, std::integral_constant<int, ahead % TW>{}, (pos + NBUF - 1) & (NBUF - 1));
+            if (left >= NBUF - 1)
+                issue(g + ahead / TW, std::integral_constant<int, ahead % TW>{}, (pos + NBUF - 1) & (NBUF - 1));
+            --left;
             pos = (pos + 1) & (NBUF - 1);
 #pragma unroll
             for (int s = 0; s < 2; ++s) {
@@ -807,7 +836,6 @@ __global__ __launch_bounds__(FMX == 1 ? 1024 : 512) void skinny_stream_kernel(co
             turn = (turn + kStreamEpoch * FMX) % waves;
         }
     }
-    wait_vm_imm<0>();  // the reloads past the last group land before the LDS is given up
 }
 
 // ---- fallback for K that is a multiple of 128 but does not split into tiles: the
@@ -1062,8 +1090,9 @@ namespace {
 // does not keep going: K up to 3072 is faster in the other form).  17 to 64 rows: 7 or 8
 // waves (256 registers each for the X fragments, TW * FMX <= 16 of them per step parity)
 // and an eight-tile ring.
-constexpr int kStreamMinGroupsPerCu = 5;       // measured crossover at up to 16 rows of X
-constexpr int kStreamMinGroupsPerCuWide = 8;   // ... with more rows of X and more than two tiles per wave
+constexpr int kStreamMinGroupsPerCu = 5;       // measured crossover at up to 16 rows of X on eight waves (K = 4096)
+constexpr int kStreamMinGroupsPerCuFull = 3;   // ... on fourteen to sixteen waves (K = 8192: 16 x 12288 x 8192 11.9 -> 10.5 us)
+constexpr int kStreamMinGroupsPerCuWide = 10;  // ... with more rows of X and more than two tiles per wave
 
 struct StreamPlan {
     int tw = 0, s = 0, fmx = 1, bufs = 4, groups_per_block = 0, grid = 0, lds = 0;
@@ -1082,7 +1111,9 @@ bool make_stream_plan(int m, int n, int k, int cu_count, StreamPlan &p)
     if (s == 0)
         return false;
     const int groups = (n + 15) / 16;
-    if (groups < (fmx == 1 || tiles / s <= 2 ? kStreamMinGroupsPerCu : kStreamMinGroupsPerCuWide) * cu_count)
+    const int min_groups = fmx == 1 ? (s >= 14 ? kStreamMinGroupsPerCuFull : kStreamMinGroupsPerCu)
+                                    : (tiles / s <= 2 ? kStreamMinGroupsPerCu : kStreamMinGroupsPerCuWide);
+    if (groups < min_groups * cu_count)
         return false;
     p.tw = tiles / s;
     p.s = s;
