@@ -29,8 +29,8 @@
 // wavefronts split K into S slices of T tiles of 256 nibbles; a wave issues every load
 // of its slices before it waits for anything, multiplies each row group as soon as it has
 // landed (loads complete in issue order, so that is a wait for a known number of younger
-// loads), adds its share to the group's block of sums in LDS and counts itself in at the
-// group's arrival counter; the wave that completes a counter stores the group.  Each wave
+// loads) and adds its share to the group's block of sums in LDS without waiting for
+// anything; the waves meet once, at the end, and store the blocks side by side.  Each wave
 // fetches its own slice of X once and reuses it for its R row groups, so larger R cuts the
 // (L2-resident, but hot-line) X traffic.  No global atomics, no workspace, and the result
 // does not depend on timing (integer additions commute).
@@ -168,10 +168,9 @@ constexpr int max_threads(int t, int r, int fmx, bool xdma)
     return (!xdma && (t * fmx > 4 || (t * fmx == 4 && r * fmx >= 8))) ? 512 : 1024;
 }
 
-// LDS in front of the waves' tiles: the arrival counters, one per row group of W, in the first
-// 16 bytes (ds_append addresses them with the instruction's 16-bit constant), and from 1 KiB
-// on one 16 x 16 block of sums (1 KiB) per pair (row group of W, row group of X).
-constexpr int head_bytes(int r, int fmx) { return 1024 + r * fmx * 1024; }
+// LDS in front of the waves' tiles: one 16 x 16 block of sums (1 KiB) per pair (row group
+// of W, row group of X).
+constexpr int head_bytes(int r, int fmx) { return r * fmx * 1024; }
 
 // T tiles per wave, R row groups per workgroup, FMX 16-row groups of X (M <= 16*FMX).
 // XDMA: X tiles go through LDS like W; otherwise they are loaded into registers in
@@ -182,7 +181,8 @@ constexpr int head_bytes(int r, int fmx) { return 1024 + r * fmx * 1024; }
 // X, rest of W; since loads complete in order, "row group rg, tile t has landed" is a wait
 // for a fixed number of younger loads.  Each row group is multiplied and added to the
 // group's sums as soon as it has landed, while the later groups are still in flight, so
-// only the last group's share is exposed after the last byte arrives.
+// only the last group's share, the meeting and the stores are exposed after the last byte
+// arrives.
 template <int T, int R, int FMX, bool XDMA, bool RAGGED>
 __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(const uint8_t *X, const uint8_t *W, int32_t *Y,
                                                                               v4i dims, Epilogue ep_all)
@@ -235,15 +235,11 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
 
     const unsigned my_lds = uniform(lds_base + kHead + wave * kWaveTiles * kTileBytes);
     // Waves take the row groups in different orders: wave w keeps group (i + w) mod R in its
-    // i-th tiles.  The last wave to arrive at a group stores it, and with one order for all
-    // the slowest wave is the last at every group and stores them all, one after the other,
-    // when everybody else has left; rotated, the groups' last arrivals fall to different
-    // waves, which store side by side (16 x 14336 x 4096: 7.5 -> 7.3 us, 64 rows: 10.7 -> 9.9).
+    // i-th tiles (measured: nothing at up to 16 rows of X, 3 % with more).
     const int rot = wave & (R - 1);
     const int himask = (int)0xF0F0F0F0u;
     const uint8_t *mine = lds + kHead + wave * kWaveTiles * kTileBytes;
-    int *const arrived = (int *)lds;
-    int *const sums = (int *)(lds + 1024);
+    int *const sums = (int *)lds;
 
     // Fragment layout: lane l supplies row l%16 and, in step s of a tile, chunk
     // 4*s + l/16 (32 nibbles: even ones feed one MFMA, odd ones the next).
@@ -264,7 +260,6 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
     // S * T tiles, each wave refills its own LDS tiles (nobody else reads them, and its own
     // reads of the previous pass have been consumed).
     int skip = 0;
-    unsigned to_store = 0;  // row groups this wave was the last to arrive at
 #pragma unroll 1
     for (int pass = 0; pass < passes; ++pass) {
     {
@@ -310,13 +305,10 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
     // rest of W.
     if (pass > 0)
         issue_w(kZero, kZero, kOne);
-    // With the first loads on their way: the arrival counters and the sums start at zero,
-    // which everybody has to have seen before anybody adds to them.  (Meeting here, where
-    // every wave is about to wait for memory anyway, measured better than meeting in front
-    // of the first addition.)
+    // With the first loads on their way: the sums start at zero, which everybody has to have
+    // seen before anybody adds to them.  (Meeting here, where every wave is about to wait for
+    // memory anyway, measured better than meeting in front of the first addition.)
     if (pass == 0) {
-        if (threadIdx.x < 4)
-            arrived[threadIdx.x] = 0;
         for (int i = threadIdx.x; i < R * FMX * 256; i += waves * 64)
             sums[i] = 0;
         __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
@@ -511,50 +503,28 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
 #pragma unroll
             for (int q = 0; q < 4; ++q)
                 __hip_atomic_fetch_add(block + f * 256 + q * 64, acc[f][q] >> 8, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        asm volatile("" ::: "memory");  // (the compiler keeps the order too)
-        // Then the wave counts itself in: ds_append adds the number of active lanes (64) to the
-        // counter, whose address is the instruction's constant (byte 4 * rg of the workgroup's
-        // LDS), and returns what was there.  A wave's LDS operations take effect in the order
-        // issued, so the wave that finds the counter complete finds all the sums complete.
-        int seen;
-        switch (rg) {
-        case 0:
-            asm volatile("s_mov_b32 m0, 0\n\tds_append %0 offset:0\n\ts_waitcnt lgkmcnt(0)" : "=v"(seen) : : "memory");
-            break;
-        case 1:
-            asm volatile("s_mov_b32 m0, 0\n\tds_append %0 offset:4\n\ts_waitcnt lgkmcnt(0)" : "=v"(seen) : : "memory");
-            break;
-        case 2:
-            asm volatile("s_mov_b32 m0, 0\n\tds_append %0 offset:8\n\ts_waitcnt lgkmcnt(0)" : "=v"(seen) : : "memory");
-            break;
-        default:
-            asm volatile("s_mov_b32 m0, 0\n\tds_append %0 offset:12\n\ts_waitcnt lgkmcnt(0)" : "=v"(seen) : : "memory");
-            break;
-        }
-        // The last wave to arrive at a group stores it, once it is through with its own groups.
-        if (__builtin_amdgcn_readfirstlane(seen) == 64 * (waves * passes - 1))
-            to_store |= 1u << rg;
     }
     }  // passes
 
-    if (to_store == 0)
-        return;
-    const int om = lane >> 2, oj = lane & 3;  // this lane stores Y[om][4 * oj ..+4) of each block
+    // ---- everybody's shares are in after one meeting; the R * FMX blocks are then stored by
+    //      as many waves, side by side.  (An arrival counter per row group, ds_append returning
+    //      its old value, with the last wave to arrive storing the group while the others were
+    //      still multiplying, was 4 % slower with several row groups and no faster with one:
+    //      every wave then waits for the counter's old value after every group.)
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    const int om = lane >> 2, oj = lane & 3;  // this lane stores Y[om][4 * oj ..+4) of a block
     if (plain && ((N | rows_here) & 3) == 0) {
         // Nothing to load or to convert, and a lane's four outputs exist together or not at
         // all: the path that ends the kernel in the common case, kept to a few instructions.
-        const int *mine_of = sums + 16 * oj + om;
-        int32_t *dst = Y + (size_t)om * N + n0 + 4 * oj;
 #pragma unroll 1
-        for (int rg = 0; rg < R; ++rg, mine_of += FMX * 256, dst += 16) {
-            if (!((to_store >> rg) & 1u))
-                continue;
-#pragma unroll
-            for (int f = 0; f < FMX; ++f) {
-                const v4i sum = {mine_of[f * 256], mine_of[f * 256 + 64], mine_of[f * 256 + 128], mine_of[f * 256 + 192]};
-                if (f * 16 + om < M && rg * 16 + 4 * oj < rows_here)
-                    *(v4i *)(dst + (size_t)f * 16 * N) = sum;
-            }
+        for (int j = wave; j < R * FMX; j += waves) {  // block j: row group j / FMX of W, j % FMX of X
+            const int rg = j / FMX, f = j % FMX;
+            const int *mine_of = sums + j * 256 + 16 * oj + om;
+            const v4i sum = {mine_of[0], mine_of[64], mine_of[128], mine_of[192]};
+            if (f * 16 + om < M && rg * 16 + 4 * oj < rows_here)
+                *(v4i *)(Y + (size_t)(f * 16 + om) * N + n0 + rg * 16 + 4 * oj) = sum;
         }
         return;
     }
@@ -562,32 +532,27 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
     Epilogue ep = ep_all;
     asm volatile("" : "+s"(ep.bias), "+s"(ep.row_scale), "+s"(ep.col_scale), "+s"(ep.f32));
 #pragma unroll 1
-    for (int rg = 0; rg < R; ++rg) {
-        if (!((to_store >> rg) & 1u))
-            continue;
+    for (int j = wave; j < R * FMX; j += waves) {
+        const int rg = j / FMX, f = j % FMX;
+        const int *mine_of = sums + j * 256 + 16 * oj + om;
+        v4i sum = {mine_of[0], mine_of[64], mine_of[128], mine_of[192]};
+        const int m = f * 16 + om;
+        const int nb = rg * 16 + 4 * oj;  // within the workgroup's rows
+        int32_t *dst = Y + (size_t)m * N + n0 + nb;
+        if (m < M) {
+            const float rs = ep.row_scale ? ep.row_scale[m] : 1.f;
 #pragma unroll
-        for (int f = 0; f < FMX; ++f) {
-            const int *mine_of = sums + (rg * FMX + f) * 256 + 16 * oj + om;
-            v4i sum = {mine_of[0], mine_of[64], mine_of[128], mine_of[192]};
-            const int m = f * 16 + om;
-            const int nb = rg * 16 + 4 * oj;  // within the workgroup's rows
-            int32_t *dst = Y + (size_t)m * N + n0 + nb;
-            if (m < M) {
-                const float rs = ep.row_scale ? ep.row_scale[m] : 1.f;
+            for (int q = 0; q < 4; ++q) {
+                const int nn = n0 + (nb + q < rows_here ? nb + q : rows_here - 1);
+                sum[q] = epilogue_value(ep, sum[q], ep.bias ? ep.bias[nn] : 0, rs, ep.col_scale ? ep.col_scale[nn] : 1.f);
+            }
+            if (nb + 3 < rows_here && (N & 3) == 0) {
+                *(v4i *)dst = sum;
+            } else {
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const int nn = n0 + (nb + q < rows_here ? nb + q : rows_here - 1);
-                    sum[q] = epilogue_value(ep, sum[q], ep.bias ? ep.bias[nn] : 0, rs,
-                                            ep.col_scale ? ep.col_scale[nn] : 1.f);
-                }
-                if (nb + 3 < rows_here && (N & 3) == 0) {
-                    *(v4i *)dst = sum;
-                } else {
-#pragma unroll
-                    for (int q = 0; q < 4; ++q)
-                        if (nb + q < rows_here)
-                            dst[q] = sum[q];
-                }
+                for (int q = 0; q < 4; ++q)
+                    if (nb + q < rows_here)
+                        dst[q] = sum[q];
             }
         }
     }
