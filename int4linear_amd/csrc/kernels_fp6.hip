@@ -244,7 +244,19 @@ struct Fp6Config {
     static_assert(CHUNKS % NWAVES == 0 && CH % 2 == 0 && CH <= 63, "loads must split evenly");
 };
 
-template <class C>
+// Parts of the kernel that a measurement build leaves out to see what they cost
+// (tests/host/fp6_ablation.cpp instantiates them; the library only ever launches kWhole).
+// The results of such a build are wrong by construction.
+enum : unsigned {
+    kWhole = 0,
+    kNoStores = 1,    // the tile is not stored
+    kNoLoads = 2,     // no global -> LDS loads after the prologue (the ring keeps its first stages)
+    kNoLdsReads = 4,  // no LDS reads after the prologue (the registers keep their first operands)
+    kSameTile = 8,    // every tile reads the operands of tile (0, 0)
+    kNoBarrier = 16,  // the waves do not meet between a stage's two units (they then race on the ring)
+};
+
+template <class C, unsigned LEFT_OUT = kWhole>
 __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
     const uint8_t *__restrict__ XW, const uint8_t *__restrict__ WW, int32_t *__restrict__ Y,
     int M, int N, int K, int tiles_m, int tiles_n, int ksplit, Epilogue ep)
@@ -288,6 +300,8 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
         const int item = bid + it * nblk;
         const int slice = item / tiles;
         tile_coords(item - slice * tiles, tiles, tiles_m, tiles_n, tm, tn);
+        if constexpr (LEFT_OUT & kSameTile)
+            tm = tn = 0;
         xptr = XW + ((size_t)tm * KT_all + (size_t)slice * KT) * kOperandStageBytes;
         wptr = WW + ((size_t)tn * KT_all + (size_t)slice * KT) * kOperandStageBytes;
     };
@@ -392,10 +406,12 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
     static_assert(kDmaFirstSlot + C::CH / 2 <= C::SLOTS, "not enough slots for the loads");
     auto spread = [&](auto slot_tag, unsigned read_ring, int read_kf, int read_p, auto half_pos, unsigned load_ring) {
         constexpr int slot = decltype(slot_tag)::value;
+        if constexpr (!(LEFT_OUT & kNoLdsReads)) {
 #pragma unroll
-        for (int r = slot * kReadsPerSlot; r < (slot + 1) * kReadsPerSlot && r < kReads; ++r)
-            read_op(read_ring, read_kf, read_p, r);
-        if constexpr (slot >= kDmaFirstSlot && slot < kDmaFirstSlot + C::CH / 2) {
+            for (int r = slot * kReadsPerSlot; r < (slot + 1) * kReadsPerSlot && r < kReads; ++r)
+                read_op(read_ring, read_kf, read_p, r);
+        }
+        if constexpr (!(LEFT_OUT & kNoLoads) && slot >= kDmaFirstSlot && slot < kDmaFirstSlot + C::CH / 2) {
             ld_chunk(std::integral_constant<int, decltype(half_pos)::value * (C::CH / 2) + slot - kDmaFirstSlot>{}, load_ring);
         }
     };
@@ -422,6 +438,11 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
 #pragma unroll
     for (int r = 0; r < kReads; ++r)
         read_op(0u, 0, 0, r);
+    if constexpr (LEFT_OUT & kNoLdsReads) {
+#pragma unroll
+        for (int r = 0; r < kReads; ++r)
+            read_op(0u, 1, 1, r);
+    }
 
     int stores_behind = 0;  // a tile has just been stored: its stores sit behind the loads waited for next
     // One iteration of the stage loop, for the stage whose buffer is ring position RING.  The
@@ -470,7 +491,8 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
                          : "scc", "memory");
             stores_behind = 0;
             __builtin_amdgcn_s_waitcnt(I4L_WAIT_LGKM0);
-            __builtin_amdgcn_s_barrier();
+            if constexpr (!(LEFT_OUT & kNoBarrier))
+                __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
         }
 
@@ -510,7 +532,9 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
                 const int ncol = ln + i * kFragRows;
                 col_off[i] = ncol < cols_left ? (unsigned)ncol * 4u : 0x40000000u;
             }
-            if (ep_plain) {
+            if constexpr (LEFT_OUT & kNoStores) {
+                pin(acc[0][0]);
+            } else if (ep_plain) {
 #pragma unroll
                 for (int j = 0; j < C::FM; ++j) {
 #pragma unroll

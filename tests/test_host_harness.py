@@ -108,3 +108,21 @@ def test_mfma_ceiling_reports_rates(gpu):
     assert r.returncode == 0, r.stdout + r.stderr
     rows = re.findall(r"\[MFMA\] (int8|fp6) .*? ([\d.]+) TOPS +([\d.]+) GHz", r.stdout)
     assert len(rows) == 8 and all(float(t) > 500 and 0.5 < float(g) < 3.0 for _, t, g in rows), r.stdout
+
+
+def test_fp6_ablation_usage_error_without_a_device():
+    r = subprocess.run([str(_binary("fp6_ablation")), "--bogus"], capture_output=True, text=True)
+    assert r.returncode == 2 and "usage" in r.stderr
+
+
+@pytest.mark.gpu
+def test_fp6_ablation_reports_every_build(gpu):
+    """The FP6 kernel with parts left out: every build runs and none is slower than the whole
+    kernel by more than noise (a small shape; the figures that matter come from 8192^3)."""
+    r = subprocess.run([str(_binary("fp6_ablation")), "2048x2048x4096", "--iters", "10", "--warmup", "5"],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout + r.stderr
+    rows = re.findall(r"\[ABLATION\] (.*?) +([\d.]+) us +([\d.]+) TOPS", r.stdout)
+    assert len(rows) == 10 and rows[0][0] == "whole kernel", r.stdout
+    whole = float(rows[0][1])
+    assert all(0 < float(us) < 1.5 * whole for _, us, _ in rows), r.stdout
