@@ -104,16 +104,27 @@ int int4linear_gemm_s4s4s32_ex(const void *a_packed_d, const void *b_packed_d, v
  * such entry point; its README lists the bias add as future work (README.md:72).
  *   int4linear_linear_s32:  Y[i][j] = sum_l X[i][l] W[j][l] + bias[j]          (int32, wraps)
  *   int4linear_linear_f32:  Y[i][j] = ((float)(sum + bias[j]) * row_scale[i]) * col_scale[j]
+ *   int4linear_linear_f16:  the same value rounded once more, to IEEE half (nearest even;
+ *                           beyond 65504 it becomes infinity)
+ *   int4linear_linear_bf16: the same value rounded once more, to bfloat16 (nearest even)
  * bias_d (n int32), row_scale_d (m floats: per-token activation scale) and col_scale_d
  * (n floats: per-output-channel weight scale) may each be NULL (0 / 1).  The integer part is
  * exact; the conversion to float rounds to nearest once and each multiplication once, in
- * the order written.  `kernel` is an INT4LINEAR_KERNEL_* value; other arguments as for
- * int4linear_gemm_s4s4s32. */
+ * the order written (the README's natural next step after the bias: dequantised output in
+ * the type the next layer takes).  y_d of the two half-width forms is m x n 16-bit elements,
+ * row-major, base 16-byte aligned like the others.  `kernel` is an INT4LINEAR_KERNEL_*
+ * value; other arguments as for int4linear_gemm_s4s4s32. */
 int int4linear_linear_s32(const void *x_packed_d, const void *w_packed_d, const int *bias_d, void *y_d,
                           int m, int n, int k, int kernel, void *stream);
 int int4linear_linear_f32(const void *x_packed_d, const void *w_packed_d, const int *bias_d,
                           const float *row_scale_d, const float *col_scale_d, float *y_d,
                           int m, int n, int k, int kernel, void *stream);
+int int4linear_linear_f16(const void *x_packed_d, const void *w_packed_d, const int *bias_d,
+                          const float *row_scale_d, const float *col_scale_d, void *y_d,
+                          int m, int n, int k, int kernel, void *stream);
+int int4linear_linear_bf16(const void *x_packed_d, const void *w_packed_d, const int *bias_d,
+                           const float *row_scale_d, const float *col_scale_d, void *y_d,
+                           int m, int n, int k, int kernel, void *stream);
 
 /* Device-side counterparts of utils/packer.cpp:3-18 (pack) and :20-31 (unpack):
  * src_d / dst_d are device arrays with the reference's host layouts (m x n ints

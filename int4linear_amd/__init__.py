@@ -12,6 +12,8 @@ from .api import (  # noqa: F401
     gemm_s4s4s32_static,
     init,
     kernel_for_shape,
+    linear_bf16,
+    linear_f16,
     linear_f32,
     linear_s32,
     linear_v0_launch,

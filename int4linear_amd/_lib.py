@@ -26,6 +26,10 @@ C_ABI = [
     ("int4linear_linear_s32", c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     ("int4linear_linear_f32", c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                       c_int, c_void_p]),
+    ("int4linear_linear_f16", c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                      c_int, c_void_p]),
+    ("int4linear_linear_bf16", c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                       c_int, c_void_p]),
     ("int4linear_fp6_operand_bytes", c_size_t, [c_int, c_int]),
     ("int4linear_fp6_convert", c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
     ("int4linear_gemm_fp6_converted", c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),

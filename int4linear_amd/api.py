@@ -86,6 +86,28 @@ def linear_f32(x_packed_d, w_packed_d, bias_d, row_scale_d, col_scale_d, y_d, m:
                                          ctypes.c_void_p(stream)))
 
 
+def linear_f16(x_packed_d, w_packed_d, bias_d, row_scale_d, col_scale_d, y_d, m: int, n: int, k: int, *,
+               kernel: str = "auto", stream: int | None = None) -> None:
+    """Y (float16) = the value of linear_f32 rounded to nearest even once more."""
+    lib = _lib.load()
+    if stream is None:
+        stream = _current_stream()
+    _lib.check(lib.int4linear_linear_f16(_ptr(x_packed_d), _ptr(w_packed_d), _ptr(bias_d), _ptr(row_scale_d),
+                                         _ptr(col_scale_d), _ptr(y_d), m, n, k, KERNELS[kernel],
+                                         ctypes.c_void_p(stream)))
+
+
+def linear_bf16(x_packed_d, w_packed_d, bias_d, row_scale_d, col_scale_d, y_d, m: int, n: int, k: int, *,
+                kernel: str = "auto", stream: int | None = None) -> None:
+    """Y (bfloat16) = the value of linear_f32 rounded to nearest even once more."""
+    lib = _lib.load()
+    if stream is None:
+        stream = _current_stream()
+    _lib.check(lib.int4linear_linear_bf16(_ptr(x_packed_d), _ptr(w_packed_d), _ptr(bias_d), _ptr(row_scale_d),
+                                          _ptr(col_scale_d), _ptr(y_d), m, n, k, KERNELS[kernel],
+                                          ctypes.c_void_p(stream)))
+
+
 def fp6_operand_bytes(rows: int, k: int) -> int:
     """Bytes of the converted (FP6) form of a rows x k operand; 0 if k is unsupported."""
     return int(_lib.load().int4linear_fp6_operand_bytes(rows, k))

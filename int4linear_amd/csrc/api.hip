@@ -288,7 +288,7 @@ int gemm_impl(const void *a, const void *b, void *c, int m, int n, int k, int ke
         return st;
     hipStream_t stream = (hipStream_t)stream_v;
 
-    const bool plain = !ep.bias && !ep.row_scale && !ep.col_scale && !ep.f32;
+    const bool plain = !ep.bias && !ep.row_scale && !ep.col_scale && !ep.out;
     if (k == 0 && plain) {
         hipError_t e = launch_zero_i32((int *)c, (size_t)m * (size_t)n, stream);
         return e == hipSuccess ? INT4LINEAR_OK : fail_hip(e);
@@ -406,7 +406,31 @@ int int4linear_linear_f32(const void *x_packed_d, const void *w_packed_d, const 
     ep.bias = bias_d;
     ep.row_scale = row_scale_d;
     ep.col_scale = col_scale_d;
-    ep.f32 = 1;
+    ep.out = kOutF32;
+    return gemm_impl(x_packed_d, w_packed_d, y_d, m, n, k, kernel, stream, ep);
+}
+
+int int4linear_linear_f16(const void *x_packed_d, const void *w_packed_d, const int *bias_d,
+                          const float *row_scale_d, const float *col_scale_d, void *y_d, int m, int n,
+                          int k, int kernel, void *stream)
+{
+    Epilogue ep;
+    ep.bias = bias_d;
+    ep.row_scale = row_scale_d;
+    ep.col_scale = col_scale_d;
+    ep.out = kOutF16;
+    return gemm_impl(x_packed_d, w_packed_d, y_d, m, n, k, kernel, stream, ep);
+}
+
+int int4linear_linear_bf16(const void *x_packed_d, const void *w_packed_d, const int *bias_d,
+                           const float *row_scale_d, const float *col_scale_d, void *y_d, int m, int n,
+                           int k, int kernel, void *stream)
+{
+    Epilogue ep;
+    ep.bias = bias_d;
+    ep.row_scale = row_scale_d;
+    ep.col_scale = col_scale_d;
+    ep.out = kOutBF16;
     return gemm_impl(x_packed_d, w_packed_d, y_d, m, n, k, kernel, stream, ep);
 }
 

@@ -8,26 +8,82 @@ namespace int4linear {
 
 // Optional work between the accumulator and the store of every output element (i, j):
 //   v = acc + bias[j]                                   (bias null: + 0)
-//   f32 == 0: C is int32 and receives v
-//   f32 != 0: C is float and receives (float)v * row_scale[i] * col_scale[j]
-//             (a null scale counts as 1; the two multiplications happen in that order)
+//   out == kOutS32: C is int32 and receives v
+//   otherwise:      t = (float)v * row_scale[i] * col_scale[j]
+//                   (a null scale counts as 1; the two multiplications happen in that order)
+//     kOutF32:  C is float and receives t
+//     kOutF16:  C is IEEE half and receives t rounded to nearest even
+//     kOutBF16: C is bfloat16 and receives t rounded to nearest even (NaN stays a quiet NaN)
 // Passed to the kernels by value; an all-zero struct is the plain GEMM.
+enum OutKind : int { kOutS32 = 0, kOutF32 = 1, kOutF16 = 2, kOutBF16 = 3 };
+
 struct Epilogue {
     const int32_t *bias = nullptr;
     const float *row_scale = nullptr;
     const float *col_scale = nullptr;
-    int f32 = 0;
+    int out = kOutS32;  // an OutKind
 };
 
 #if defined(__HIPCC__)
-// The 32 bits stored for one output element.
+// The bits stored for one output element: 32 of them, or 16 in the low half for the two
+// half-width kinds.
 __device__ __forceinline__ int epilogue_value(const Epilogue &ep, int acc, int bias_j, float row_scale_i,
                                               float col_scale_j)
 {
     const int v = acc + bias_j;
-    if (!ep.f32)
+    if (!ep.out)
         return v;
-    return __float_as_int(((float)v * row_scale_i) * col_scale_j);
+    const float t = ((float)v * row_scale_i) * col_scale_j;
+    if (ep.out == kOutF32)
+        return __float_as_int(t);
+    if (ep.out == kOutF16)
+        return (int)(unsigned short)__builtin_bit_cast(unsigned short, (_Float16)t);
+    const unsigned bits = (unsigned)__float_as_int(t);
+    if ((bits & 0x7fffffffu) > 0x7f800000u)
+        return (int)((bits >> 16) | 0x0040u);
+    return (int)((bits + 0x7fffu + ((bits >> 16) & 1u)) >> 16);
+}
+
+__device__ __forceinline__ bool out_is_half_width(const Epilogue &ep) { return ep.out >= kOutF16; }
+
+// Element `index` of the output array, whichever its width.
+__device__ __forceinline__ void store_out(const Epilogue &ep, void *c, size_t index, int bits)
+{
+    if (out_is_half_width(ep))
+        ((unsigned short *)c)[index] = (unsigned short)bits;
+    else
+        ((int *)c)[index] = bits;
+}
+
+// Four consecutive outputs of one row, elements index .. index + 3, of which the first `valid`
+// (0 .. 4) exist.  `together`: all four exist and index is a multiple of four elements from a
+// 16-byte-aligned base with a row length that is one too, so they go out as one store.
+typedef int out_v4i __attribute__((ext_vector_type(4)));
+typedef int out_v2i __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void store_out4(const Epilogue &ep, void *c, size_t index, out_v4i bits, int valid,
+                                           bool together)
+{
+    if (out_is_half_width(ep)) {
+        unsigned short *dst = (unsigned short *)c + index;
+        if (together) {
+            *(out_v2i *)dst = (out_v2i){bits[0] | (bits[1] << 16), bits[2] | (bits[3] << 16)};
+        } else {
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                if (q < valid)
+                    dst[q] = (unsigned short)bits[q];
+        }
+    } else {
+        int *dst = (int *)c + index;
+        if (together) {
+            *(out_v4i *)dst = bits;
+        } else {
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                if (q < valid)
+                    dst[q] = bits[q];
+        }
+    }
 }
 #endif
 

@@ -277,7 +277,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
     const int total_tiles = tiles * ksplit;  // work items
     const int nblk = gridDim.x;
     const int bid = blockIdx.x;
-    const bool ep_plain = ksplit > 1 || (!ep.bias && !ep.row_scale && !ep.col_scale && !ep.f32);
+    const bool ep_plain = ksplit > 1 || (!ep.bias && !ep.row_scale && !ep.col_scale && !ep.out);
     if (bid >= total_tiles)
         return;
     const int my_tiles = (total_tiles - bid + nblk - 1) / nblk;
@@ -562,6 +562,15 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
                     bias_v[i] = ep.bias ? ep.bias[nn] : 0;
                     cs_v[i] = ep.col_scale ? ep.col_scale[nn] : 1.f;
                 }
+                // The output may be half as wide: its own descriptor and offsets, in elements
+                // of `esz` bytes (no K-slices here: an epilogue goes with ksplit == 1).
+                const unsigned esz = out_is_half_width(ep) ? 2u : 4u;
+                __amdgpu_buffer_rsrc_t rsrc_out = __builtin_amdgcn_make_buffer_rsrc(
+                    (uint8_t *)Y + ((size_t)m0 * N + n0) * esz, 0, (int)(extent / 4u * esz), 0x00020000);
+                unsigned col_out[C::FN];
+#pragma unroll
+                for (int i = 0; i < C::FN; ++i)
+                    col_out[i] = col_off[i] == 0x40000000u ? 0x40000000u : col_off[i] / 4u * esz;
 #pragma unroll
                 for (int j = 0; j < C::FM; ++j) {
                     float rs[16];
@@ -573,11 +582,14 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
 #pragma unroll
                     for (int t = 0; t < 16; ++t) {
                         const int dm = j * kFragRows + 8 * (t / 4) + (t % 4);  // uniform
-                        const unsigned row_off = lm + dm < rows_left ? lm_off + (unsigned)dm * (unsigned)N * 4u : 0x80000000u;
+                        const unsigned row_off = lm + dm < rows_left ? (unsigned)(lm + dm) * (unsigned)N * esz : 0x80000000u;
 #pragma unroll
                         for (int i = 0; i < C::FN; ++i) {
                             const int v = epilogue_value(ep, (int)(acc[i][j][t] * kUnscale), bias_v[i], rs[t], cs_v[i]);
-                            __builtin_amdgcn_raw_buffer_store_b32((unsigned)v, rsrc, row_off + col_off[i], 0, 2 /* nt */);
+                            if (esz == 2u)
+                                __builtin_amdgcn_raw_buffer_store_b16((unsigned short)v, rsrc_out, row_off + col_out[i], 0, 2 /* nt */);
+                            else
+                                __builtin_amdgcn_raw_buffer_store_b32((unsigned)v, rsrc_out, row_off + col_out[i], 0, 2 /* nt */);
                         }
                     }
                 }

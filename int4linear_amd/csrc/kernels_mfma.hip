@@ -151,7 +151,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
     const int total_tiles = tiles_m * tiles_n * ksplit;  // work items
     const int nblk = gridDim.x;
     const int bid = blockIdx.x;
-    const bool ep_plain = ksplit > 1 || (!ep.bias && !ep.row_scale && !ep.col_scale && !ep.f32);
+    const bool ep_plain = ksplit > 1 || (!ep.bias && !ep.row_scale && !ep.col_scale && !ep.out);
     if (bid >= total_tiles)
         return;
     const int my_tiles = (total_tiles - bid + nblk - 1) / nblk;
@@ -537,6 +537,15 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
                     bias_v[i] = ep.bias ? ep.bias[nn] : 0;
                     cs_v[i] = ep.col_scale ? ep.col_scale[nn] : 1.f;
                 }
+                // The output may be half as wide: its own descriptor and offsets, in elements
+                // of `esz` bytes (no K-slices here: an epilogue goes with ksplit == 1).
+                const unsigned esz = out_is_half_width(ep) ? 2u : 4u;
+                __amdgpu_buffer_rsrc_t rsrc_out = __builtin_amdgcn_make_buffer_rsrc(
+                    (uint8_t *)Y + ((size_t)m0 * N + n0) * esz, 0, (int)(extent / 4u * esz), 0x00020000);
+                unsigned col_out[C::FN];
+#pragma unroll
+                for (int i = 0; i < C::FN; ++i)
+                    col_out[i] = col_off[i] == 0x40000000u ? 0x40000000u : col_off[i] / 4u * esz;
 #pragma unroll
                 for (int j = 0; j < C::FM; ++j) {
                     float rs[16];
@@ -548,11 +557,14 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
 #pragma unroll
                     for (int t = 0; t < 16; ++t) {
                         const int dm = j * kFrag + 8 * (t / 4) + (t % 4);  // uniform
-                        const unsigned row_off = lm + dm < rows_left ? lm_off + (unsigned)dm * (unsigned)N * 4u : 0x80000000u;
+                        const unsigned row_off = lm + dm < rows_left ? (unsigned)(lm + dm) * (unsigned)N * esz : 0x80000000u;
 #pragma unroll
                         for (int i = 0; i < C::FN; ++i) {
                             const int v = epilogue_value(ep, acc[i][j][t] >> 8, bias_v[i], rs[t], cs_v[i]);
-                            __builtin_amdgcn_raw_buffer_store_b32((unsigned)v, rsrc, row_off + col_off[i], 0, kStoreAux);
+                            if (esz == 2u)
+                                __builtin_amdgcn_raw_buffer_store_b16((unsigned short)v, rsrc_out, row_off + col_out[i], 0, kStoreAux);
+                            else
+                                __builtin_amdgcn_raw_buffer_store_b32((unsigned)v, rsrc_out, row_off + col_out[i], 0, kStoreAux);
                         }
                     }
                 }
@@ -822,7 +834,8 @@ __global__ __launch_bounds__(512) void mfma_pair_kernel(const uint8_t *__restric
     const int mw = m0 + wm * 64 + 4 * (lane >> 5);
     const int nw = n0 + wn * 64 + (lane & 31);
     int32_t *out = Y + (size_t)mw * N + nw;
-    if (ksplit > 1 || (!ep.bias && !ep.row_scale && !ep.col_scale && !ep.f32)) {
+    unsigned short *out16 = (unsigned short *)Y + ((size_t)mw * N + nw);  // the same element of a half-width output
+    if (ksplit > 1 || (!ep.bias && !ep.row_scale && !ep.col_scale && !ep.out)) {
         // nothing to load: the stores follow one another without a wait
 #pragma unroll
         for (int j = 0; j < 2; ++j)
@@ -857,8 +870,13 @@ __global__ __launch_bounds__(512) void mfma_pair_kernel(const uint8_t *__restric
             const int dm = 32 * j + 8 * (t / 4) + (t % 4);
 #pragma unroll
             for (int i = 0; i < 2; ++i)
-                if (mw + dm < M && nw + 32 * i < N)
-                    out[(size_t)dm * N + 32 * i] = epilogue_value(ep, acc[i][j][t], bias_v[i], rs[t], cs_v[i]);
+                if (mw + dm < M && nw + 32 * i < N) {
+                    const int v = epilogue_value(ep, acc[i][j][t], bias_v[i], rs[t], cs_v[i]);
+                    if (out_is_half_width(ep))  // (no K-slices here: Y is the output's base)
+                        out16[(size_t)dm * N + 32 * i] = (unsigned short)v;
+                    else
+                        out[(size_t)dm * N + 32 * i] = v;
+                }
         }
     }
 }
@@ -964,7 +982,8 @@ __global__ __launch_bounds__(512) void mfma_pair64_kernel(const uint8_t *__restr
     const int mw = m0 + wm * kFrag + 4 * (lane >> 5);
     const int nw = n0 + wn * kFrag + (lane & 31);
     int32_t *out = Y + (size_t)mw * N + nw;
-    if (ksplit > 1 || (!ep.bias && !ep.row_scale && !ep.col_scale && !ep.f32)) {
+    unsigned short *out16 = (unsigned short *)Y + ((size_t)mw * N + nw);  // the same element of a half-width output
+    if (ksplit > 1 || (!ep.bias && !ep.row_scale && !ep.col_scale && !ep.out)) {
 #pragma unroll
         for (int t = 0; t < 16; ++t) {
             const int dm = 8 * (t / 4) + (t % 4);
@@ -983,8 +1002,13 @@ __global__ __launch_bounds__(512) void mfma_pair64_kernel(const uint8_t *__restr
 #pragma unroll
     for (int t = 0; t < 16; ++t) {
         const int dm = 8 * (t / 4) + (t % 4);
-        if (mw + dm < M && nw < N)
-            out[(size_t)dm * N] = epilogue_value(ep, acc[t], bias_v, rs[t], cs_v);
+        if (mw + dm < M && nw < N) {
+            const int v = epilogue_value(ep, acc[t], bias_v, rs[t], cs_v);
+            if (out_is_half_width(ep))  // (no K-slices here: Y is the output's base)
+                out16[(size_t)dm * N] = (unsigned short)v;
+            else
+                out[(size_t)dm * N] = v;
+        }
     }
 }
 

@@ -50,9 +50,9 @@ __global__ __launch_bounds__(kTile *kTile) void simple_gemm_kernel(
         __syncthreads();
     }
     if (row < m && col < n)
-        c[row * n + col] = epilogue_value(ep, acc, ep.bias ? ep.bias[col] : 0,
-                                          ep.row_scale ? ep.row_scale[row] : 1.f,
-                                          ep.col_scale ? ep.col_scale[col] : 1.f);
+        store_out(ep, c, (size_t)(row * n + col),
+                  epilogue_value(ep, acc, ep.bias ? ep.bias[col] : 0, ep.row_scale ? ep.row_scale[row] : 1.f,
+                                 ep.col_scale ? ep.col_scale[col] : 1.f));
 }
 
 // utils/packer.cpp:3-18 on device arrays: one thread per destination word.
@@ -97,6 +97,7 @@ __global__ void zero_i32_kernel(int4 *__restrict__ dst4, int *__restrict__ dst, 
 }
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
 
 // Second kernel of the split-K forms: Y = epilogue(sum of the ksplit slabs), four outputs of
 // one row per thread (VEC: n % 4 == 0) or one.
@@ -127,10 +128,16 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const int32_t *__res
 #pragma unroll
     for (int q = 0; q < kPer; ++q)
         sum[q] = epilogue_value(ep, sum[q], ep.bias ? ep.bias[col + q] : 0, rs, ep.col_scale ? ep.col_scale[col + q] : 1.f);
-    if constexpr (VEC)
+    if (out_is_half_width(ep)) {
+        if constexpr (VEC)  // i % 4 == 0: four half-width outputs are eight aligned bytes
+            *(v2i *)((unsigned short *)Y + i) = (v2i){sum[0] | (sum[1] << 16), sum[2] | (sum[3] << 16)};
+        else
+            ((unsigned short *)Y)[i] = (unsigned short)sum[0];
+    } else if constexpr (VEC) {
         *(v4i *)(Y + i) = (v4i){sum[0], sum[1], sum[2], sum[3]};
-    else
+    } else {
         Y[i] = sum[0];
+    }
 }
 
 }  // namespace

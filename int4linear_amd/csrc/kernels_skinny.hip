@@ -530,7 +530,7 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
     }
     // (the epilogue's operands are first looked at here, not ahead of the loads)
     Epilogue ep = ep_all;
-    asm volatile("" : "+s"(ep.bias), "+s"(ep.row_scale), "+s"(ep.col_scale), "+s"(ep.f32));
+    asm volatile("" : "+s"(ep.bias), "+s"(ep.row_scale), "+s"(ep.col_scale), "+s"(ep.out));
 #pragma unroll 1
     for (int j = wave; j < R * FMX; j += waves) {
         const int rg = j / FMX, f = j % FMX;
@@ -538,7 +538,6 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
         v4i sum = {mine_of[0], mine_of[64], mine_of[128], mine_of[192]};
         const int m = f * 16 + om;
         const int nb = rg * 16 + 4 * oj;  // within the workgroup's rows
-        int32_t *dst = Y + (size_t)m * N + n0 + nb;
         if (m < M) {
             const float rs = ep.row_scale ? ep.row_scale[m] : 1.f;
 #pragma unroll
@@ -546,14 +545,7 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
                 const int nn = n0 + (nb + q < rows_here ? nb + q : rows_here - 1);
                 sum[q] = epilogue_value(ep, sum[q], ep.bias ? ep.bias[nn] : 0, rs, ep.col_scale ? ep.col_scale[nn] : 1.f);
             }
-            if (nb + 3 < rows_here && (N & 3) == 0) {
-                *(v4i *)dst = sum;
-            } else {
-#pragma unroll
-                for (int q = 0; q < 4; ++q)
-                    if (nb + q < rows_here)
-                        dst[q] = sum[q];
-            }
+            store_out4(ep, Y, (size_t)m * N + n0 + nb, sum, rows_here - nb, nb + 3 < rows_here && ((N | n0) & 3) == 0);
         }
     }
 }
@@ -787,15 +779,7 @@ __global__ __launch_bounds__(FMX == 1 ? 1024 : 512) void skinny_stream_kernel(co
                         sum[q] = epilogue_value(ep, sum[q], ep.bias ? ep.bias[nn] : 0, rs,
                                                 ep.col_scale ? ep.col_scale[nn] : 1.f);
                     }
-                    int32_t *dst = Y + (size_t)m * N + n;
-                    if (n + 3 < N && (N & 3) == 0) {
-                        *(v4i *)dst = sum;
-                    } else {
-#pragma unroll
-                        for (int q = 0; q < 4; ++q)
-                            if (n + q < N)
-                                dst[q] = sum[q];
-                    }
+                    store_out4(ep, Y, (size_t)m * N + n, sum, N - n, n + 3 < N && (N & 3) == 0);
                 }
             }
             turn = (turn + kStreamEpoch * FMX) % waves;
@@ -864,15 +848,7 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_basic_kernel(
                 s[q] = epilogue_value(ep, s[q], ep.bias ? ep.bias[nn] : 0, rs,
                                       ep.col_scale ? ep.col_scale[nn] : 1.f);
             }
-            int32_t *dst = Y + (size_t)m * N + n;
-            if (n + 3 < N && (N & 3) == 0) {
-                *(v4i *)dst = s;
-            } else {
-#pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    if (n + t < N)
-                        dst[t] = s[t];
-            }
+            store_out4(ep, Y, (size_t)m * N + n, s, N - n, n + 3 < N && (N & 3) == 0);
         }
     }
 }
@@ -988,7 +964,7 @@ hipError_t launch_plan(const Plan &p, const void *a, const void *b, void *c, int
     if (p.s == 0)  // set-up call: raise the dynamic-LDS limit of this instantiation
         return hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
     const unsigned grid = (unsigned)((n + p.rows_blk - 1) / p.rows_blk);
-    const int plain = !ep.bias && !ep.row_scale && !ep.col_scale && !ep.f32;
+    const int plain = !ep.bias && !ep.row_scale && !ep.col_scale && !ep.out;
     // More than 16 * FMX rows of X go out in runs of that many, one launch each (the rows of
     // W are then streamed again, through the caches they were just pulled through).
     for (int m0 = 0; m0 < m; m0 += 16 * FMX) {
@@ -997,7 +973,7 @@ hipError_t launch_plan(const Plan &p, const void *a, const void *b, void *c, int
             run_ep.row_scale += m0;
         const int rows = m - m0 < 16 * FMX ? m - m0 : 16 * FMX;
         kern<<<grid, p.s * 64, p.lds, stream>>>((const uint8_t *)a + (size_t)m0 * (size_t)(k >> 1), (const uint8_t *)b,
-                                                (int32_t *)c + (size_t)m0 * (size_t)n,
+                                                (int32_t *)((uint8_t *)c + (size_t)m0 * (size_t)n * (ep.out >= kOutF16 ? 2u : 4u)),
                                                 (v4i){rows | (p.passes << 8) | (p.s << 16) | (plain << 24), n, k, p.rows_blk}, run_ep);
         const hipError_t e = hipGetLastError();
         if (e != hipSuccess)

@@ -24,6 +24,11 @@
  *                        bias, float32 astype / multiply (IEEE round-to-nearest, same
  *                        order) for the scaled output, plus the identities
  *                        "no operands == the plain product" and "scales of 1 == cast".
+ *                        The two half-width outputs (oracle_f32_to_f16_bits,
+ *                        oracle_f32_to_bf16_bits: one more rounding to nearest even) are
+ *                        pinned against numpy's float16 conversion over every float16 value,
+ *                        every halfway point between neighbours and random floats, and
+ *                        against torch's bfloat16 conversion likewise.
  */
 #include <stddef.h>
 #include <stdint.h>
@@ -113,6 +118,57 @@ int oracle_is_same(const int *a, const int *b, int count)
  * product y (m x n): v = y[i][j] + bias[j] (two's-complement wrap), and for f32 != 0
  * the 32 bits of ((float)v * row_scale[i]) * col_scale[j].  Null operands count as 0 / 1.
  * Compiled without floating-point contraction; the two products round separately. */
+/* float -> IEEE half, round to nearest even; beyond the largest half it is infinity, a NaN
+ * becomes the quiet NaN 0x7e00 with the sign kept. */
+unsigned oracle_f32_to_f16_bits(float f)
+{
+    union { float f; uint32_t u; } v;
+    v.f = f;
+    const uint32_t sign = (v.u >> 16) & 0x8000u;
+    const uint32_t x = v.u & 0x7fffffffu;
+    if (x > 0x7f800000u)
+        return sign | 0x7e00u;
+    if (x >= 0x47800000u) /* 65536 and up, infinity included */
+        return sign | 0x7c00u;
+    if (x >= 0x38800000u) { /* at least 2^-14: a normal half unless the rounding carries into infinity */
+        uint32_t h = (((x >> 23) - 112u) << 10) | ((x & 0x7fffffu) >> 13);
+        const uint32_t rem = x & 0x1fffu;
+        if (rem > 0x1000u || (rem == 0x1000u && (h & 1u)))
+            ++h;
+        return sign | h;
+    }
+    if (x < 0x33000000u) /* below 2^-25: nearer to zero than to the smallest subnormal (2^-25 itself ties to even) */
+        return sign;
+    {
+        const uint32_t mant = (x & 0x7fffffu) | 0x800000u;
+        const unsigned shift = 126u - (x >> 23); /* 14 .. 24: the result counts units of 2^-24 */
+        uint32_t h = mant >> shift;
+        const uint32_t rem = mant & ((1u << shift) - 1u), halfway = 1u << (shift - 1u);
+        if (rem > halfway || (rem == halfway && (h & 1u)))
+            ++h;
+        return sign | h;
+    }
+}
+
+/* float -> bfloat16 (the upper half of the float), round to nearest even; a NaN keeps its
+ * upper half and becomes quiet. */
+unsigned oracle_f32_to_bf16_bits(float f)
+{
+    union { float f; uint32_t u; } v;
+    v.f = f;
+    if ((v.u & 0x7fffffffu) > 0x7f800000u)
+        return (v.u >> 16) | 0x0040u;
+    return (v.u + 0x7fffu + ((v.u >> 16) & 1u)) >> 16;
+}
+
+/* n floats to half (kind 2) or bfloat16 (kind 3) bit patterns. */
+void oracle_convert_f32(const float *src, unsigned short *dst, size_t n, int kind)
+{
+    for (size_t i = 0; i < n; ++i)
+        dst[i] = (unsigned short)(kind == 2 ? oracle_f32_to_f16_bits(src[i]) : oracle_f32_to_bf16_bits(src[i]));
+}
+
+/* `out`: 0 int32, 1 float32 (its bits), 2 half, 3 bfloat16 (16 bits in the low half of the int). */
 void oracle_epilogue(int *y, int m, int n, const int *bias, const float *row_scale,
                      const float *col_scale, int f32)
 {
@@ -126,7 +182,7 @@ void oracle_epilogue(int *y, int m, int n, const int *bias, const float *row_sca
                 const float f = a * (col_scale ? col_scale[j] : 1.0f);
                 union { float f; int i; } u;
                 u.f = f;
-                v = u.i;
+                v = f32 == 2 ? (int)oracle_f32_to_f16_bits(f) : f32 == 3 ? (int)oracle_f32_to_bf16_bits(f) : u.i;
             }
             y[(size_t)i * n + j] = v;
         }

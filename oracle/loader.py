@@ -91,11 +91,16 @@ def linear_ref(x: np.ndarray, w: np.ndarray, threads: int = 1) -> np.ndarray:
     return y
 
 
-def epilogue(y: np.ndarray, bias=None, row_scale=None, col_scale=None, f32: bool = False) -> np.ndarray:
-    """Applies the linear layer's epilogue to an int32 product; returns int32, or float32
-    when f32 is set."""
-    out = np.ascontiguousarray(_i32(y)).copy()
-    m, n = out.shape
+OUT_KINDS = {"s32": 0, "f32": 1, "f16": 2, "bf16": 3}
+
+
+def epilogue(y: np.ndarray, bias=None, row_scale=None, col_scale=None, f32: bool = False, out: str | None = None) -> np.ndarray:
+    """Applies the linear layer's epilogue to an int32 product; returns int32, float32 (f32 set
+    or out == "f32"), or the uint16 bit patterns of the half / bfloat16 output (out == "f16",
+    "bf16")."""
+    kind = OUT_KINDS[out] if out is not None else (1 if f32 else 0)
+    buf = np.ascontiguousarray(_i32(y)).copy()
+    m, n = buf.shape
     keep = []
 
     def ptr(a, dtype, count):
@@ -110,9 +115,23 @@ def epilogue(y: np.ndarray, bias=None, row_scale=None, col_scale=None, f32: bool
     fn.restype = None
     fn.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                    ctypes.c_int]
-    fn(out.ctypes.data, m, n, ptr(bias, np.int32, n), ptr(row_scale, np.float32, m), ptr(col_scale, np.float32, n),
-       1 if f32 else 0)
-    return out.view(np.float32) if f32 else out
+    fn(buf.ctypes.data, m, n, ptr(bias, np.int32, n), ptr(row_scale, np.float32, m), ptr(col_scale, np.float32, n),
+       kind)
+    if kind >= 2:
+        return buf.astype(np.uint16)
+    return buf.view(np.float32) if kind == 1 else buf
+
+
+def convert_f32(values: np.ndarray, out: str) -> np.ndarray:
+    """float32 values to the uint16 bit patterns of half ("f16") or bfloat16 ("bf16"), as the
+    epilogue rounds them."""
+    src = np.ascontiguousarray(values, dtype=np.float32).ravel()
+    dst = np.empty(src.size, dtype=np.uint16)
+    fn = oracle().oracle_convert_f32
+    fn.restype = None
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+    fn(src.ctypes.data, dst.ctypes.data, src.size, OUT_KINDS[out])
+    return dst.reshape(np.shape(values))
 
 
 def is_same(a: np.ndarray, b: np.ndarray) -> bool:

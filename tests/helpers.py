@@ -69,3 +69,22 @@ def to_device_bytes(packed: np.ndarray):
     import torch
 
     return torch.from_numpy(np.ascontiguousarray(packed).view(np.uint8).reshape(-1)).to("cuda:0")
+
+
+def check_half_width_outputs(xd, wd, want: np.ndarray, bias: np.ndarray, rs: np.ndarray, cs: np.ndarray,
+                             m: int, n: int, k: int, kernel: str = "auto") -> None:
+    """linear_f16 / linear_bf16 on device operands against the oracle's epilogue of the int32
+    product `want`, bit for bit, with the row scales shrunk so that most outputs stay inside
+    the half range; the elements behind the m x n outputs must stay untouched."""
+    import torch
+
+    import int4linear_amd as lib
+
+    rs_small = (rs * np.float32(2.0 ** -9)).astype(np.float32)
+    bd, rd, cd = (torch.from_numpy(a).to("cuda:0") for a in (bias, rs_small, cs))
+    for kind, fn in (("f16", lib.linear_f16), ("bf16", lib.linear_bf16)):
+        y16 = torch.full((m * n + 256,), 0x7BAD, dtype=torch.int16, device="cuda:0")
+        fn(xd, wd, bd, rd, cd, y16, m, n, k, kernel=kernel)
+        got = y16.cpu().numpy().view(np.uint16)
+        assert np.array_equal(got[:m * n].reshape(m, n), oracle.epilogue(want, bias, rs_small, cs, out=kind)), f"{kind} {kernel}"
+        assert np.all(got[m * n:] == 0x7BAD), f"{kind} {kernel}: wrote past the output"

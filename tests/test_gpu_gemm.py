@@ -208,6 +208,10 @@ def test_linear_with_epilogue(gpu, host_threads, m, n, k, kernels):
     xd = helpers.to_device_bytes(helpers.pack_bytes(x))
     wd = helpers.to_device_bytes(helpers.pack_bytes(w))
     bd, rd, cd = (torch.from_numpy(a).to("cuda:0") for a in (bias, rs, cs))
+    rs_small = (rs * np.float32(2.0 ** -9)).astype(np.float32)   # keeps most outputs inside the half range
+    rd_small = torch.from_numpy(rs_small).to("cuda:0")
+    want_16 = {kind: oracle.epilogue(prod, bias, rs_small, cs, out=kind) for kind in ("f16", "bf16")}
+    plain_16 = {kind: oracle.epilogue(prod, None, None, None, out=kind) for kind in ("f16", "bf16")}
     for kern in kernels:
         y = torch.full((m, n), 0x7BADBAD, dtype=torch.int32, device="cuda:0")
         lib.linear_s32(xd, wd, bd, y, m, n, k, kernel=kern)
@@ -220,6 +224,16 @@ def test_linear_with_epilogue(gpu, host_threads, m, n, k, kernels):
         assert np.array_equal(yf.cpu().numpy().view(np.int32), want_f32.view(np.int32)), f"f32 {kern}"
         lib.linear_f32(xd, wd, None, rd, None, yf, m, n, k, kernel=kern)
         assert np.array_equal(yf.cpu().numpy().view(np.int32), want_f32_nobias.view(np.int32)), f"f32 row scale {kern}"
+        # half-width outputs: the same value rounded once more; the elements behind the m x n
+        # outputs stay untouched (a store of the wrong width would reach them)
+        for kind, fn in (("f16", lib.linear_f16), ("bf16", lib.linear_bf16)):
+            y16 = torch.full((m * n + 256,), 0x7BAD, dtype=torch.int16, device="cuda:0")
+            fn(xd, wd, bd, rd_small, cd, y16, m, n, k, kernel=kern)
+            got = y16.cpu().numpy().view(np.uint16)
+            assert np.array_equal(got[:m * n].reshape(m, n), want_16[kind]), f"{kind} {kern}"
+            assert np.all(got[m * n:] == 0x7BAD), f"{kind} {kern}: wrote past the output"
+            fn(xd, wd, None, None, None, y16, m, n, k, kernel=kern)
+            assert np.array_equal(y16.cpu().numpy().view(np.uint16)[:m * n].reshape(m, n), plain_16[kind]), f"{kind} plain {kern}"
 
 
 def test_internal_workspace_shared_between_streams(gpu, host_threads):
@@ -278,6 +292,7 @@ def test_small_grid_form_of_the_int8_kernel(gpu, host_threads, m, n, k):
     assert np.array_equal(yf.cpu().numpy().view(np.int32), oracle.epilogue(want, bias, rs, cs, f32=True).view(np.int32))
     lib.linear_f32(xd, wd, None, rd, None, yf, m, n, k, kernel="mfma")
     assert np.array_equal(yf.cpu().numpy().view(np.int32), oracle.epilogue(want, None, rs, None, f32=True).view(np.int32))
+    helpers.check_half_width_outputs(xd, wd, want, bias, rs, cs, m, n, k, kernel="mfma")
 
 
 @pytest.mark.parametrize("m, n, k", [(300, 2049, 8192), (257, 1000, 4096), (512, 1024, 14336), (300, 520, 16392),
@@ -312,6 +327,7 @@ def test_split_k_form_of_the_fp6_kernel(gpu, host_threads, m, n, k):
     yf = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda:0")
     lib.linear_f32(xd, wd, bd, rd, cd, yf, m, n, k, kernel="fp6")
     assert np.array_equal(yf.cpu().numpy().view(np.int32), oracle.epilogue(want, bias, rs, cs, f32=True).view(np.int32))
+    helpers.check_half_width_outputs(xd, wd, want, bias, rs, cs, m, n, k, kernel="fp6")
 
 
 @pytest.mark.parametrize("m, n, k", [(128, 4096, 14336), (300, 520, 12288), (1024, 512, 14336), (100, 300, 8192),
@@ -344,6 +360,7 @@ def test_split_k_form_of_the_int8_kernel(gpu, host_threads, m, n, k):
     yf = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda:0")
     lib.linear_f32(xd, wd, bd, rd, cd, yf, m, n, k)
     assert np.array_equal(yf.cpu().numpy().view(np.int32), oracle.epilogue(want, bias, rs, cs, f32=True).view(np.int32))
+    helpers.check_half_width_outputs(xd, wd, want, bias, rs, cs, m, n, k)
     # without a workspace the same call runs unsplit
     lib.set_workspace_limit(0)
     try:

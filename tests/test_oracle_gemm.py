@@ -133,3 +133,63 @@ def test_epilogue_against_numpy():
     # only one of the scales
     assert np.array_equal(oracle.epilogue(y, None, rs, None, f32=True), y.astype(np.float32) * rs[:, None])
     assert np.array_equal(oracle.epilogue(y, None, None, cs, f32=True), y.astype(np.float32) * cs[None, :])
+
+
+def _interesting_floats(rng):
+    """Every float16 value as a float, every midpoint between float16 neighbours, the floats
+    next to those midpoints, and random bit patterns (NaNs left out)."""
+    h = np.arange(0x10000, dtype=np.uint16).view(np.float16).astype(np.float32)
+    h = h[np.isfinite(h)]
+    hs = np.sort(np.unique(h))
+    mid = ((hs[:-1].astype(np.float64) + hs[1:].astype(np.float64)) / 2).astype(np.float32)  # exact in float32
+    near = np.concatenate([np.nextafter(mid, np.float32(np.inf)), np.nextafter(mid, np.float32(-np.inf))])
+    big = np.array([65504.0, 65519.99, 65520.0, 65520.01, 65536.0, 1e6, 3.4e38, np.inf, 2.0**-24, 2.0**-25,
+                    np.nextafter(np.float32(2.0**-25), np.float32(1)), 2.0**-26, 0.0], dtype=np.float32)
+    big = np.concatenate([big, -big])
+    rnd = rng.integers(0, 2**32, size=200000, dtype=np.uint64).astype(np.uint32).view(np.float32)
+    rnd = rnd[~np.isnan(rnd)]
+    return np.concatenate([h, mid, near, big, rnd])
+
+
+def test_half_conversion_against_numpy():
+    """float -> half as the epilogue rounds it: numpy's conversion (round to nearest even,
+    overflow to infinity, gradual underflow) is the independent implementation."""
+    v = _interesting_floats(np.random.default_rng(21))
+    with np.errstate(over="ignore"):
+        want = v.astype(np.float16).view(np.uint16)
+    got = oracle.convert_f32(v, "f16")
+    assert np.array_equal(got, want), np.flatnonzero(got != want)[:5]
+
+
+def test_bfloat16_conversion_against_torch():
+    """float -> bfloat16: torch's CPU conversion is the independent implementation; the closed
+    form (exactly representable values, ties to even on the 17th bit) is checked as well."""
+    import torch
+
+    v = _interesting_floats(np.random.default_rng(22))
+    bits = v.view(np.uint32)
+    ties = ((bits & 0xFFFF0000) | 0x8000).view(np.float32)       # exact halfway points
+    v = np.concatenate([v, ties[np.isfinite(ties)]])
+    want = torch.from_numpy(v.copy()).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    got = oracle.convert_f32(v, "bf16")
+    assert np.array_equal(got, want), np.flatnonzero(got != want)[:5]
+    exact = (np.arange(0x7F80, dtype=np.uint32) << 16).view(np.float32)   # every finite bfloat16 value
+    assert np.array_equal(oracle.convert_f32(exact, "bf16"), np.arange(0x7F80, dtype=np.uint16))
+    assert oracle.convert_f32(np.array([1.00390625], np.float32), "bf16")[0] == 0x3F80       # 1 + 2^-8 ties down to even
+    assert oracle.convert_f32(np.array([1.01171875], np.float32), "bf16")[0] == 0x3F82       # 1 + 3 * 2^-8 ties up to even
+
+
+def test_epilogue_half_width_outputs():
+    rng = np.random.default_rng(23)
+    m, n = 19, 37
+    y = rng.integers(-2**22, 2**22, size=(m, n), dtype=np.int32)
+    bias = rng.integers(-2**10, 2**10, size=n, dtype=np.int32)
+    rs = rng.uniform(0.0001, 0.01, size=m).astype(np.float32)
+    cs = rng.uniform(0.001, 3.0, size=n).astype(np.float32)
+    f = oracle.epilogue(y, bias, rs, cs, out="f32")
+    for kind in ("f16", "bf16"):
+        got = oracle.epilogue(y, bias, rs, cs, out=kind)
+        assert got.dtype == np.uint16 and got.shape == (m, n)
+        assert np.array_equal(got, oracle.convert_f32(f, kind))
+    with np.errstate(over="ignore"):
+        assert np.array_equal(oracle.epilogue(y, bias, rs, cs, out="f16"), f.astype(np.float16).view(np.uint16))
