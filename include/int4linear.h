@@ -107,6 +107,8 @@ int int4linear_gemm_s4s4s32_ex(const void *a_packed_d, const void *b_packed_d, v
  *   int4linear_linear_f16:  the same value rounded once more, to IEEE half (nearest even;
  *                           beyond 65504 it becomes infinity)
  *   int4linear_linear_bf16: the same value rounded once more, to bfloat16 (nearest even)
+ *                           (both: denormals are kept; a NaN, which only a scale can bring
+ *                           in, keeps its sign and upper payload bits and becomes quiet)
  * bias_d (n int32), row_scale_d (m floats: per-token activation scale) and col_scale_d
  * (n floats: per-output-channel weight scale) may each be NULL (0 / 1).  The integer part is
  * exact; the conversion to float rounds to nearest once and each multiplication once, in

@@ -3,6 +3,9 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#if defined(__HIPCC__)
+#include <type_traits>
+#endif
 
 namespace int4linear {
 
@@ -13,7 +16,9 @@ namespace int4linear {
 //                   (a null scale counts as 1; the two multiplications happen in that order)
 //     kOutF32:  C is float and receives t
 //     kOutF16:  C is IEEE half and receives t rounded to nearest even
-//     kOutBF16: C is bfloat16 and receives t rounded to nearest even (NaN stays a quiet NaN)
+//     kOutBF16: C is bfloat16 and receives t rounded to nearest even
+//     (both: t is a float first, so there are two roundings; overflow goes to infinity,
+//     denormals are kept, a NaN keeps its sign and upper payload bits and becomes quiet)
 // Passed to the kernels by value; an all-zero struct is the plain GEMM.
 enum OutKind : int { kOutS32 = 0, kOutF32 = 1, kOutF16 = 2, kOutBF16 = 3 };
 
@@ -25,23 +30,40 @@ struct Epilogue {
 };
 
 #if defined(__HIPCC__)
-// The bits stored for one output element: 32 of them, or 16 in the low half for the two
-// half-width kinds.
-__device__ __forceinline__ int epilogue_value(const Epilogue &ep, int acc, int bias_j, float row_scale_i,
-                                              float col_scale_j)
+// The 32 bits stored for one output element of the two full-width kinds.
+__device__ __forceinline__ int epilogue_value32(const Epilogue &ep, int acc, int bias_j, float row_scale_i,
+                                                float col_scale_j)
 {
     const int v = acc + bias_j;
     if (!ep.out)
         return v;
-    const float t = ((float)v * row_scale_i) * col_scale_j;
-    if (ep.out == kOutF32)
-        return __float_as_int(t);
+    return __float_as_int(((float)v * row_scale_i) * col_scale_j);
+}
+
+// The 16 bits (in the low half) stored for one output element of the two half-width kinds.
+__device__ __forceinline__ int epilogue_value16(const Epilogue &ep, int acc, int bias_j, float row_scale_i,
+                                                float col_scale_j)
+{
+    float t = ((float)(acc + bias_j) * row_scale_i) * col_scale_j;
+    // The product is rounded to float before it is rounded to 16 bits; with the product in
+    // sight the compiler would merge the two into one instruction that rounds once
+    // (v_fma_mixlo_f16), which differs at ties.
+    asm("" : "+v"(t));
     if (ep.out == kOutF16)
         return (int)(unsigned short)__builtin_bit_cast(unsigned short, (_Float16)t);
-    const unsigned bits = (unsigned)__float_as_int(t);
-    if ((bits & 0x7fffffffu) > 0x7f800000u)
-        return (int)((bits >> 16) | 0x0040u);
-    return (int)((bits + 0x7fffu + ((bits >> 16) & 1u)) >> 16);
+    // gfx950 converts in hardware (v_cvt_pk_bf16_f32): round to nearest even, denormals kept,
+    // a NaN keeps its sign and its upper payload bits and becomes quiet.
+    return (int)__builtin_bit_cast(unsigned short, (__bf16)t);
+}
+
+__device__ __forceinline__ bool out_is_half_width(const Epilogue &ep);
+
+// Either of them, by the kind of output.
+__device__ __forceinline__ int epilogue_value(const Epilogue &ep, int acc, int bias_j, float row_scale_i,
+                                              float col_scale_j)
+{
+    return ep.out >= kOutF16 ? epilogue_value16(ep, acc, bias_j, row_scale_i, col_scale_j)
+                             : epilogue_value32(ep, acc, bias_j, row_scale_i, col_scale_j);
 }
 
 __device__ __forceinline__ bool out_is_half_width(const Epilogue &ep) { return ep.out >= kOutF16; }
@@ -58,12 +80,13 @@ __device__ __forceinline__ void store_out(const Epilogue &ep, void *c, size_t in
 // Four consecutive outputs of one row, elements index .. index + 3, of which the first `valid`
 // (0 .. 4) exist.  `together`: all four exist and index is a multiple of four elements from a
 // 16-byte-aligned base with a row length that is one too, so they go out as one store.
+// HALF: the output's elements are 16 bits wide.
 typedef int out_v4i __attribute__((ext_vector_type(4)));
 typedef int out_v2i __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ void store_out4(const Epilogue &ep, void *c, size_t index, out_v4i bits, int valid,
-                                           bool together)
+template <bool HALF>
+__device__ __forceinline__ void store_out4(void *c, size_t index, out_v4i bits, int valid, bool together)
 {
-    if (out_is_half_width(ep)) {
+    if constexpr (HALF) {
         unsigned short *dst = (unsigned short *)c + index;
         if (together) {
             *(out_v2i *)dst = (out_v2i){bits[0] | (bits[1] << 16), bits[2] | (bits[3] << 16)};
@@ -84,6 +107,27 @@ __device__ __forceinline__ void store_out4(const Epilogue &ep, void *c, size_t i
                     dst[q] = bits[q];
         }
     }
+}
+
+template <bool HALF>
+__device__ __forceinline__ int epilogue_value_of(const Epilogue &ep, int acc, int bias_j, float row_scale_i,
+                                                 float col_scale_j)
+{
+    if constexpr (HALF)
+        return epilogue_value16(ep, acc, bias_j, row_scale_i, col_scale_j);
+    else
+        return epilogue_value32(ep, acc, bias_j, row_scale_i, col_scale_j);
+}
+
+// f(std::true_type) for the half-width kinds of output, f(std::false_type) for the others:
+// the kind is looked at once, not per element.
+template <class F>
+__device__ __forceinline__ void by_output_width(const Epilogue &ep, F &&f)
+{
+    if (out_is_half_width(ep))
+        f(std::true_type{});
+    else
+        f(std::false_type{});
 }
 #endif
 

@@ -256,7 +256,9 @@ enum : unsigned {
     kNoBarrier = 16,  // the waves do not meet between a stage's two units (they then race on the ring)
 };
 
-template <class C, unsigned LEFT_OUT = kWhole>
+// HALF_OUT: the build for the two output kinds of 16-bit elements (its own build, so that the
+// one for 32-bit elements carries none of its code).
+template <class C, unsigned LEFT_OUT = kWhole, bool HALF_OUT = false>
 __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
     const uint8_t *__restrict__ XW, const uint8_t *__restrict__ WW, int32_t *__restrict__ Y,
     int M, int N, int K, int tiles_m, int tiles_n, int ksplit, Epilogue ep)
@@ -277,7 +279,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
     const int total_tiles = tiles * ksplit;  // work items
     const int nblk = gridDim.x;
     const int bid = blockIdx.x;
-    const bool ep_plain = ksplit > 1 || (!ep.bias && !ep.row_scale && !ep.col_scale && !ep.out);
+    const bool ep_plain = !HALF_OUT && (ksplit > 1 || (!ep.bias && !ep.row_scale && !ep.col_scale && !ep.out));
     if (bid >= total_tiles)
         return;
     const int my_tiles = (total_tiles - bid + nblk - 1) / nblk;
@@ -562,34 +564,50 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
                     bias_v[i] = ep.bias ? ep.bias[nn] : 0;
                     cs_v[i] = ep.col_scale ? ep.col_scale[nn] : 1.f;
                 }
-                // The output may be half as wide: its own descriptor and offsets, in elements
-                // of `esz` bytes (no K-slices here: an epilogue goes with ksplit == 1).
-                const unsigned esz = out_is_half_width(ep) ? 2u : 4u;
-                __amdgpu_buffer_rsrc_t rsrc_out = __builtin_amdgcn_make_buffer_rsrc(
-                    (uint8_t *)Y + ((size_t)m0 * N + n0) * esz, 0, (int)(extent / 4u * esz), 0x00020000);
-                unsigned col_out[C::FN];
+                if constexpr (!HALF_OUT) {
 #pragma unroll
-                for (int i = 0; i < C::FN; ++i)
-                    col_out[i] = col_off[i] == 0x40000000u ? 0x40000000u : col_off[i] / 4u * esz;
+                    for (int j = 0; j < C::FM; ++j) {
+                        float rs[16];
 #pragma unroll
-                for (int j = 0; j < C::FM; ++j) {
-                    float rs[16];
+                        for (int t = 0; t < 16; ++t) {
+                            const int dm = j * kFragRows + 8 * (t / 4) + (t % 4);
+                            rs[t] = ep.row_scale ? ep.row_scale[m0 + (lm + dm < rows_left ? lm + dm : rows_left - 1)] : 1.f;
+                        }
 #pragma unroll
-                    for (int t = 0; t < 16; ++t) {
-                        const int dm = j * kFragRows + 8 * (t / 4) + (t % 4);
-                        rs[t] = ep.row_scale ? ep.row_scale[m0 + (lm + dm < rows_left ? lm + dm : rows_left - 1)] : 1.f;
+                        for (int t = 0; t < 16; ++t) {
+                            const int dm = j * kFragRows + 8 * (t / 4) + (t % 4);  // uniform
+                            const unsigned row_off = lm + dm < rows_left ? lm_off + (unsigned)dm * (unsigned)N * 4u : 0x80000000u;
+#pragma unroll
+                            for (int i = 0; i < C::FN; ++i) {
+                                const int v = epilogue_value32(ep, (int)(acc[i][j][t] * kUnscale), bias_v[i], rs[t], cs_v[i]);
+                                __builtin_amdgcn_raw_buffer_store_b32((unsigned)v, rsrc, row_off + col_off[i], 0, 2 /* nt */);
+                            }
+                        }
                     }
+                } else {
+                    // The half-width kinds: a descriptor over the same tile of an output of
+                    // two-byte elements, every offset halved (no K-slices here: an epilogue
+                    // goes with ksplit == 1, Y is the output's base).
+                    __amdgpu_buffer_rsrc_t rsrc16 = __builtin_amdgcn_make_buffer_rsrc(
+                        (uint8_t *)Y + ((size_t)m0 * N + n0) * 2u, 0, (int)(extent / 2u), 0x00020000);
 #pragma unroll
-                    for (int t = 0; t < 16; ++t) {
-                        const int dm = j * kFragRows + 8 * (t / 4) + (t % 4);  // uniform
-                        const unsigned row_off = lm + dm < rows_left ? (unsigned)(lm + dm) * (unsigned)N * esz : 0x80000000u;
+                    for (int j = 0; j < C::FM; ++j) {
+                        float rs[16];
 #pragma unroll
-                        for (int i = 0; i < C::FN; ++i) {
-                            const int v = epilogue_value(ep, (int)(acc[i][j][t] * kUnscale), bias_v[i], rs[t], cs_v[i]);
-                            if (esz == 2u)
-                                __builtin_amdgcn_raw_buffer_store_b16((unsigned short)v, rsrc_out, row_off + col_out[i], 0, 2 /* nt */);
-                            else
-                                __builtin_amdgcn_raw_buffer_store_b32((unsigned)v, rsrc_out, row_off + col_out[i], 0, 2 /* nt */);
+                        for (int t = 0; t < 16; ++t) {
+                            const int dm = j * kFragRows + 8 * (t / 4) + (t % 4);
+                            rs[t] = ep.row_scale ? ep.row_scale[m0 + (lm + dm < rows_left ? lm + dm : rows_left - 1)] : 1.f;
+                        }
+#pragma unroll
+                        for (int t = 0; t < 16; ++t) {
+                            const int dm = j * kFragRows + 8 * (t / 4) + (t % 4);  // uniform
+                            const unsigned row_off = lm + dm < rows_left ? (lm_off + (unsigned)dm * (unsigned)N * 4u) / 2u : 0x80000000u;
+#pragma unroll
+                            for (int i = 0; i < C::FN; ++i) {
+                                const int v = epilogue_value16(ep, (int)(acc[i][j][t] * kUnscale), bias_v[i], rs[t], cs_v[i]);
+                                __builtin_amdgcn_raw_buffer_store_b16((unsigned short)v, rsrc16,
+                                                                      row_off + (col_off[i] == 0x40000000u ? col_off[i] : col_off[i] / 2u), 0, 2 /* nt */);
+                            }
                         }
                     }
                 }
@@ -659,7 +677,11 @@ hipError_t fp6_init(const DeviceInfo &dev)
 {
     if (dev.lds_per_cu < kLdsBytes)
         return hipErrorInvalidConfiguration;
-    return hipFuncSetAttribute((const void *)fp6_gemm_kernel<Fp6Cfg>,
+    hipError_t e = hipFuncSetAttribute((const void *)fp6_gemm_kernel<Fp6Cfg>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+    if (e != hipSuccess)
+        return e;
+    return hipFuncSetAttribute((const void *)fp6_gemm_kernel<Fp6Cfg, kWhole, true>,
                                hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
 }
 
@@ -713,8 +735,15 @@ hipError_t launch_gemm_items(const void *a_conv, const void *b_conv, void *c, in
     long grid = (long)dev.cu_count * C::OCC;
     if (grid > total)
         grid = total;
-    fp6_gemm_kernel<C><<<(unsigned)grid, C::THREADS, kLdsBytes, stream>>>(
-        (const uint8_t *)a_conv, (const uint8_t *)b_conv, (int32_t *)c, m, n, padded_k(k), tiles_m, tiles_n, ksplit, ep);
+    if (ep.out >= kOutF16) {
+        if (ksplit != 1)
+            return hipErrorInvalidValue;
+        fp6_gemm_kernel<C, kWhole, true><<<(unsigned)grid, C::THREADS, kLdsBytes, stream>>>(
+            (const uint8_t *)a_conv, (const uint8_t *)b_conv, (int32_t *)c, m, n, padded_k(k), tiles_m, tiles_n, ksplit, ep);
+    } else {
+        fp6_gemm_kernel<C><<<(unsigned)grid, C::THREADS, kLdsBytes, stream>>>(
+            (const uint8_t *)a_conv, (const uint8_t *)b_conv, (int32_t *)c, m, n, padded_k(k), tiles_m, tiles_n, ksplit, ep);
+    }
     return hipGetLastError();
 }
 

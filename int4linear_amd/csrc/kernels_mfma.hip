@@ -537,34 +537,50 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
                     bias_v[i] = ep.bias ? ep.bias[nn] : 0;
                     cs_v[i] = ep.col_scale ? ep.col_scale[nn] : 1.f;
                 }
-                // The output may be half as wide: its own descriptor and offsets, in elements
-                // of `esz` bytes (no K-slices here: an epilogue goes with ksplit == 1).
-                const unsigned esz = out_is_half_width(ep) ? 2u : 4u;
-                __amdgpu_buffer_rsrc_t rsrc_out = __builtin_amdgcn_make_buffer_rsrc(
-                    (uint8_t *)Y + ((size_t)m0 * N + n0) * esz, 0, (int)(extent / 4u * esz), 0x00020000);
-                unsigned col_out[C::FN];
+                if (!out_is_half_width(ep)) {
 #pragma unroll
-                for (int i = 0; i < C::FN; ++i)
-                    col_out[i] = col_off[i] == 0x40000000u ? 0x40000000u : col_off[i] / 4u * esz;
+                    for (int j = 0; j < C::FM; ++j) {
+                        float rs[16];
 #pragma unroll
-                for (int j = 0; j < C::FM; ++j) {
-                    float rs[16];
+                        for (int t = 0; t < 16; ++t) {
+                            const int dm = j * kFrag + 8 * (t / 4) + (t % 4);
+                            rs[t] = ep.row_scale ? ep.row_scale[m0 + (lm + dm < rows_left ? lm + dm : rows_left - 1)] : 1.f;
+                        }
 #pragma unroll
-                    for (int t = 0; t < 16; ++t) {
-                        const int dm = j * kFrag + 8 * (t / 4) + (t % 4);
-                        rs[t] = ep.row_scale ? ep.row_scale[m0 + (lm + dm < rows_left ? lm + dm : rows_left - 1)] : 1.f;
+                        for (int t = 0; t < 16; ++t) {
+                            const int dm = j * kFrag + 8 * (t / 4) + (t % 4);  // uniform
+                            const unsigned row_off = lm + dm < rows_left ? lm_off + (unsigned)dm * (unsigned)N * 4u : 0x80000000u;
+#pragma unroll
+                            for (int i = 0; i < C::FN; ++i) {
+                                const int v = epilogue_value32(ep, acc[i][j][t] >> 8, bias_v[i], rs[t], cs_v[i]);
+                                __builtin_amdgcn_raw_buffer_store_b32((unsigned)v, rsrc, row_off + col_off[i], 0, kStoreAux);
+                            }
+                        }
                     }
+                } else {
+                    // The half-width kinds: a descriptor over the same tile of an output of
+                    // two-byte elements, every offset halved (no K-slices here: an epilogue
+                    // goes with ksplit == 1, Y is the output's base).
+                    __amdgpu_buffer_rsrc_t rsrc16 = __builtin_amdgcn_make_buffer_rsrc(
+                        (uint8_t *)Y + ((size_t)m0 * N + n0) * 2u, 0, (int)(extent / 2u), 0x00020000);
 #pragma unroll
-                    for (int t = 0; t < 16; ++t) {
-                        const int dm = j * kFrag + 8 * (t / 4) + (t % 4);  // uniform
-                        const unsigned row_off = lm + dm < rows_left ? (unsigned)(lm + dm) * (unsigned)N * esz : 0x80000000u;
+                    for (int j = 0; j < C::FM; ++j) {
+                        float rs[16];
 #pragma unroll
-                        for (int i = 0; i < C::FN; ++i) {
-                            const int v = epilogue_value(ep, acc[i][j][t] >> 8, bias_v[i], rs[t], cs_v[i]);
-                            if (esz == 2u)
-                                __builtin_amdgcn_raw_buffer_store_b16((unsigned short)v, rsrc_out, row_off + col_out[i], 0, kStoreAux);
-                            else
-                                __builtin_amdgcn_raw_buffer_store_b32((unsigned)v, rsrc_out, row_off + col_out[i], 0, kStoreAux);
+                        for (int t = 0; t < 16; ++t) {
+                            const int dm = j * kFrag + 8 * (t / 4) + (t % 4);
+                            rs[t] = ep.row_scale ? ep.row_scale[m0 + (lm + dm < rows_left ? lm + dm : rows_left - 1)] : 1.f;
+                        }
+#pragma unroll
+                        for (int t = 0; t < 16; ++t) {
+                            const int dm = j * kFrag + 8 * (t / 4) + (t % 4);  // uniform
+                            const unsigned row_off = lm + dm < rows_left ? (lm_off + (unsigned)dm * (unsigned)N * 4u) / 2u : 0x80000000u;
+#pragma unroll
+                            for (int i = 0; i < C::FN; ++i) {
+                                const int v = epilogue_value16(ep, acc[i][j][t] >> 8, bias_v[i], rs[t], cs_v[i]);
+                                __builtin_amdgcn_raw_buffer_store_b16((unsigned short)v, rsrc16,
+                                                                      row_off + (col_off[i] == 0x40000000u ? col_off[i] : col_off[i] / 2u), 0, kStoreAux);
+                            }
                         }
                     }
                 }
@@ -600,8 +616,10 @@ constexpr int kPairRounds = 2;  // used up to this many tiles per CU (two workgr
 // DEEP: the widening of a stage is interleaved with the MFMAs of the stage before it, from a
 // second set of widened operands (187 registers: one workgroup per CU); otherwise it follows
 // them (110 registers: two workgroups fit a CU, and their waves fill each other's gaps).
-template <bool DEEP>
-__global__ __launch_bounds__(512) void mfma_pair_kernel(const uint8_t *__restrict__ X,
+// HALF_OUT: the build for the two output kinds of 16-bit elements (a build of its own, so
+// that the one for 32-bit elements carries none of its code or registers).
+template <bool DEEP, bool HALF_OUT = false>
+__global__ __launch_bounds__(512, DEEP ? 2 : 4) void mfma_pair_kernel(const uint8_t *__restrict__ X,
                                                         const uint8_t *__restrict__ W,
                                                         int32_t *__restrict__ Y, int M, int N, int K,
                                                         int tiles_m, int tiles_n, int ksplit, Epilogue ep)
@@ -827,15 +845,22 @@ __global__ __launch_bounds__(512) void mfma_pair_kernel(const uint8_t *__restric
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < 2; ++j) {
 #pragma unroll
             for (int t = 0; t < 16; ++t)
                 acc[i][j][t] = (acc[i][j][t] + merge[((i * 2 + j) * 16 + t) * 64]) >> 8;  // both operands carried a factor 16 (exact per slice: every product is a multiple of 256)
+            if constexpr (HALF_OUT) {  // the sums stay here: moved down to their uses, all 64 reads ahead of them do not fit the registers of this build
+#pragma unroll
+                for (int t = 0; t < 16; ++t)
+                    acc[i][j][t] = opaque(acc[i][j][t]);
+            }
+        }
     const int mw = m0 + wm * 64 + 4 * (lane >> 5);
     const int nw = n0 + wn * 64 + (lane & 31);
     int32_t *out = Y + (size_t)mw * N + nw;
-    unsigned short *out16 = (unsigned short *)Y + ((size_t)mw * N + nw);  // the same element of a half-width output
-    if (ksplit > 1 || (!ep.bias && !ep.row_scale && !ep.col_scale && !ep.out)) {
+    // a half-width output as a whole (launch_mfma sends at most a few hundred tiles here)
+    __amdgpu_buffer_rsrc_t rsrc16 = __builtin_amdgcn_make_buffer_rsrc(Y, 0, (int)((unsigned)M * (unsigned)N * 2u), 0x00020000);
+    if (!HALF_OUT && (ksplit > 1 || (!ep.bias && !ep.row_scale && !ep.col_scale && !ep.out))) {
         // nothing to load: the stores follow one another without a wait
 #pragma unroll
         for (int j = 0; j < 2; ++j)
@@ -859,24 +884,47 @@ __global__ __launch_bounds__(512) void mfma_pair_kernel(const uint8_t *__restric
         bias_v[i] = ep.bias ? ep.bias[nn] : 0;
         cs_v[i] = ep.col_scale ? ep.col_scale[nn] : 1.f;
     }
+    constexpr bool half_width = HALF_OUT;  // (no K-slices there: Y is the output's base)
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         float rs[16];
 #pragma unroll
         for (int t = 0; t < 16; ++t)
             rs[t] = ep.row_scale ? ep.row_scale[min(mw + 32 * j + 8 * (t / 4) + (t % 4), M - 1)] : 1.f;
+        if constexpr (!half_width) {
+            // The values first (opaque: they stay here), then the stores, each behind nothing
+            // but its bounds test: a value computed behind the test makes every store wait
+            // for the one before it.
+            int v[2][16];
 #pragma unroll
-        for (int t = 0; t < 16; ++t) {
-            const int dm = 32 * j + 8 * (t / 4) + (t % 4);
+            for (int t = 0; t < 16; ++t)
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
-                if (mw + dm < M && nw + 32 * i < N) {
-                    const int v = epilogue_value(ep, acc[i][j][t], bias_v[i], rs[t], cs_v[i]);
-                    if (out_is_half_width(ep))  // (no K-slices here: Y is the output's base)
-                        out16[(size_t)dm * N + 32 * i] = (unsigned short)v;
-                    else
-                        out[(size_t)dm * N + 32 * i] = v;
+                for (int i = 0; i < 2; ++i)
+                    v[i][t] = opaque(epilogue_value32(ep, acc[i][j][t], bias_v[i], rs[t], cs_v[i]));
+#pragma unroll
+            for (int t = 0; t < 16; ++t) {
+                const int dm = 32 * j + 8 * (t / 4) + (t % 4);
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+                    if (mw + dm < M && nw + 32 * i < N)
+                        out[(size_t)dm * N + 32 * i] = v[i][t];
+            }
+        } else {
+            // Stores through a descriptor over the whole output (this form only runs where
+            // it is a few MiB): an element outside the matrix gets an offset beyond it and the
+            // hardware drops the store, so there is no branch and no 64-bit address per store.
+#pragma unroll
+            for (int t = 0; t < 16; ++t) {
+                const int dm = 32 * j + 8 * (t / 4) + (t % 4);
+                const unsigned row_off = mw + dm < M ? (unsigned)(mw + dm) * (unsigned)N * 2u : 0x80000000u;
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    const unsigned col_off = nw + 32 * i < N ? (unsigned)(nw + 32 * i) * 2u : 0x40000000u;
+                    __builtin_amdgcn_raw_buffer_store_b16(
+                        (unsigned short)epilogue_value16(ep, acc[i][j][t], bias_v[i], rs[t], cs_v[i]), rsrc16,
+                        row_off + col_off, 0, 0);
                 }
+            }
         }
     }
 }
@@ -889,6 +937,7 @@ constexpr int kTinyTile = 64;
 constexpr int kTinyStageBytes = 2 * kTinyTile * kRowBytes;    // 8 KiB
 constexpr int kTinyLdsBytes = kPairStages * kTinyStageBytes;  // 32 KiB; the merge takes 16 KiB of it
 
+template <bool HALF_OUT = false>
 __global__ __launch_bounds__(512) void mfma_pair64_kernel(const uint8_t *__restrict__ X,
                                                           const uint8_t *__restrict__ W,
                                                           int32_t *__restrict__ Y, int M, int N, int K,
@@ -982,8 +1031,9 @@ __global__ __launch_bounds__(512) void mfma_pair64_kernel(const uint8_t *__restr
     const int mw = m0 + wm * kFrag + 4 * (lane >> 5);
     const int nw = n0 + wn * kFrag + (lane & 31);
     int32_t *out = Y + (size_t)mw * N + nw;
-    unsigned short *out16 = (unsigned short *)Y + ((size_t)mw * N + nw);  // the same element of a half-width output
-    if (ksplit > 1 || (!ep.bias && !ep.row_scale && !ep.col_scale && !ep.out)) {
+    // a half-width output as a whole (launch_mfma sends at most a few hundred tiles here)
+    __amdgpu_buffer_rsrc_t rsrc16 = __builtin_amdgcn_make_buffer_rsrc(Y, 0, (int)((unsigned)M * (unsigned)N * 2u), 0x00020000);
+    if (!HALF_OUT && (ksplit > 1 || (!ep.bias && !ep.row_scale && !ep.col_scale && !ep.out))) {
 #pragma unroll
         for (int t = 0; t < 16; ++t) {
             const int dm = 8 * (t / 4) + (t % 4);
@@ -999,15 +1049,27 @@ __global__ __launch_bounds__(512) void mfma_pair64_kernel(const uint8_t *__restr
 #pragma unroll
     for (int t = 0; t < 16; ++t)
         rs[t] = ep.row_scale ? ep.row_scale[min(mw + 8 * (t / 4) + (t % 4), M - 1)] : 1.f;
+    constexpr bool half_width = HALF_OUT;  // (no K-slices there: Y is the output's base)
+    if constexpr (!half_width) {
+        int v[16];  // the values first (opaque: they stay here), then the stores, each behind nothing but its bounds test
 #pragma unroll
-    for (int t = 0; t < 16; ++t) {
-        const int dm = 8 * (t / 4) + (t % 4);
-        if (mw + dm < M && nw < N) {
-            const int v = epilogue_value(ep, acc[t], bias_v, rs[t], cs_v);
-            if (out_is_half_width(ep))  // (no K-slices here: Y is the output's base)
-                out16[(size_t)dm * N] = (unsigned short)v;
-            else
-                out[(size_t)dm * N] = v;
+        for (int t = 0; t < 16; ++t)
+            v[t] = opaque(epilogue_value32(ep, acc[t], bias_v, rs[t], cs_v));
+#pragma unroll
+        for (int t = 0; t < 16; ++t) {
+            const int dm = 8 * (t / 4) + (t % 4);
+            if (mw + dm < M && nw < N)
+                out[(size_t)dm * N] = v[t];
+        }
+    } else {
+        // (stores through a descriptor over the whole output, as in mfma_pair_kernel)
+        const unsigned col_off = nw < N ? (unsigned)nw * 2u : 0x40000000u;
+#pragma unroll
+        for (int t = 0; t < 16; ++t) {
+            const int dm = 8 * (t / 4) + (t % 4);
+            const unsigned row_off = mw + dm < M ? (unsigned)(mw + dm) * (unsigned)N * 2u : 0x80000000u;
+            __builtin_amdgcn_raw_buffer_store_b16((unsigned short)epilogue_value16(ep, acc[t], bias_v, rs[t], cs_v),
+                                                  rsrc16, row_off + col_off, 0, 0);
         }
     }
 }
@@ -1129,7 +1191,7 @@ hipError_t launch_mfma_splitk(const void *a, const void *b, void *c, int m, int 
         for (int q = 2; q <= d; ++q)
             if (stages % q == 0 && (long)tiny_m * tiny_n * q <= (long)dev.cu_count * 2)
                 dt = q;
-        mfma_pair64_kernel<<<(unsigned)(tiny_m * tiny_n * dt), 512, kTinyLdsBytes, stream>>>(
+        mfma_pair64_kernel<false><<<(unsigned)(tiny_m * tiny_n * dt), 512, kTinyLdsBytes, stream>>>(
             (const uint8_t *)a, (const uint8_t *)b, (int32_t *)workspace, m, n, k, tiny_m, tiny_n, dt, Epilogue{});
         const hipError_t e2 = hipGetLastError();
         if (e2 != hipSuccess)
@@ -1160,17 +1222,20 @@ hipError_t launch_mfma(const void *a, const void *b, void *c, int m, int n, int 
     // than cu_count / 2 tiles of 128 x 128 the larger tile wins).
     if ((long)pair_m * pair_n * 2 <= dev.cu_count) {
         const int tiny_m = (m + kTinyTile - 1) / kTinyTile, tiny_n = (n + kTinyTile - 1) / kTinyTile;
-        mfma_pair64_kernel<<<(unsigned)(tiny_m * tiny_n), 512, kTinyLdsBytes, stream>>>(
-            (const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k, tiny_m, tiny_n, 1, ep);
+        if (ep.out >= kOutF16)
+            mfma_pair64_kernel<true><<<(unsigned)(tiny_m * tiny_n), 512, kTinyLdsBytes, stream>>>(
+                (const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k, tiny_m, tiny_n, 1, ep);
+        else
+            mfma_pair64_kernel<false><<<(unsigned)(tiny_m * tiny_n), 512, kTinyLdsBytes, stream>>>(
+                (const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k, tiny_m, tiny_n, 1, ep);
         return hipGetLastError();
     }
     if ((long)pair_m * pair_n <= (long)dev.cu_count * kPairRounds) {
-        if ((long)pair_m * pair_n <= dev.cu_count)
-            mfma_pair_kernel<true><<<(unsigned)(pair_m * pair_n), 512, kPairLdsBytes, stream>>>(
-                (const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k, pair_m, pair_n, 1, ep);
-        else
-            mfma_pair_kernel<false><<<(unsigned)(pair_m * pair_n), 512, kPairLdsBytes, stream>>>(
-                (const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k, pair_m, pair_n, 1, ep);
+        const bool deep = (long)pair_m * pair_n <= dev.cu_count, half_out = ep.out >= kOutF16;
+        auto *kern = deep ? (half_out ? mfma_pair_kernel<true, true> : mfma_pair_kernel<true, false>)
+                          : (half_out ? mfma_pair_kernel<false, true> : mfma_pair_kernel<false, false>);
+        kern<<<(unsigned)(pair_m * pair_n), 512, kPairLdsBytes, stream>>>(
+            (const uint8_t *)a, (const uint8_t *)b, (int32_t *)c, m, n, k, pair_m, pair_n, 1, ep);
         return hipGetLastError();
     }
     // Use the big tile once it alone can occupy every CU.

@@ -125,19 +125,20 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const int32_t *__res
     const size_t row = i / (size_t)N;
     const int col = (int)(i - row * (size_t)N);
     const float rs = ep.row_scale ? ep.row_scale[row] : 1.f;
+    by_output_width(ep, [&](auto half) {
 #pragma unroll
-    for (int q = 0; q < kPer; ++q)
-        sum[q] = epilogue_value(ep, sum[q], ep.bias ? ep.bias[col + q] : 0, rs, ep.col_scale ? ep.col_scale[col + q] : 1.f);
-    if (out_is_half_width(ep)) {
-        if constexpr (VEC)  // i % 4 == 0: four half-width outputs are eight aligned bytes
+        for (int q = 0; q < kPer; ++q)
+            sum[q] = epilogue_value_of<half()>(ep, sum[q], ep.bias ? ep.bias[col + q] : 0, rs,
+                                               ep.col_scale ? ep.col_scale[col + q] : 1.f);
+        if constexpr (half() && VEC)  // i % 4 == 0: four half-width outputs are eight aligned bytes
             *(v2i *)((unsigned short *)Y + i) = (v2i){sum[0] | (sum[1] << 16), sum[2] | (sum[3] << 16)};
-        else
+        else if constexpr (half())
             ((unsigned short *)Y)[i] = (unsigned short)sum[0];
-    } else if constexpr (VEC) {
-        *(v4i *)(Y + i) = (v4i){sum[0], sum[1], sum[2], sum[3]};
-    } else {
-        Y[i] = sum[0];
-    }
+        else if constexpr (VEC)
+            *(v4i *)(Y + i) = (v4i){sum[0], sum[1], sum[2], sum[3]};
+        else
+            Y[i] = sum[0];
+    });
 }
 
 }  // namespace

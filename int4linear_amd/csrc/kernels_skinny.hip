@@ -540,12 +540,14 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
         const int nb = rg * 16 + 4 * oj;  // within the workgroup's rows
         if (m < M) {
             const float rs = ep.row_scale ? ep.row_scale[m] : 1.f;
+            by_output_width(ep, [&](auto half) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int nn = n0 + (nb + q < rows_here ? nb + q : rows_here - 1);
-                sum[q] = epilogue_value(ep, sum[q], ep.bias ? ep.bias[nn] : 0, rs, ep.col_scale ? ep.col_scale[nn] : 1.f);
-            }
-            store_out4(ep, Y, (size_t)m * N + n0 + nb, sum, rows_here - nb, nb + 3 < rows_here && ((N | n0) & 3) == 0);
+                for (int q = 0; q < 4; ++q) {
+                    const int nn = n0 + (nb + q < rows_here ? nb + q : rows_here - 1);
+                    sum[q] = epilogue_value_of<half()>(ep, sum[q], ep.bias ? ep.bias[nn] : 0, rs, ep.col_scale ? ep.col_scale[nn] : 1.f);
+                }
+                store_out4<half()>(Y, (size_t)m * N + n0 + nb, sum, rows_here - nb, nb + 3 < rows_here && ((N | n0) & 3) == 0);
+            });
         }
     }
 }
@@ -773,13 +775,15 @@ __global__ __launch_bounds__(FMX == 1 ? 1024 : 512) void skinny_stream_kernel(co
                 const int m = 16 * f + om, n = 16 * gj + 4 * oj;
                 if (m < M) {
                     const float rs = ep.row_scale ? ep.row_scale[m] : 1.f;
+                    by_output_width(ep, [&](auto half) {
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const int nn = n + q < N ? n + q : N - 1;
-                        sum[q] = epilogue_value(ep, sum[q], ep.bias ? ep.bias[nn] : 0, rs,
-                                                ep.col_scale ? ep.col_scale[nn] : 1.f);
-                    }
-                    store_out4(ep, Y, (size_t)m * N + n, sum, N - n, n + 3 < N && (N & 3) == 0);
+                        for (int q = 0; q < 4; ++q) {
+                            const int nn = n + q < N ? n + q : N - 1;
+                            sum[q] = epilogue_value_of<half()>(ep, sum[q], ep.bias ? ep.bias[nn] : 0, rs,
+                                                               ep.col_scale ? ep.col_scale[nn] : 1.f);
+                        }
+                        store_out4<half()>(Y, (size_t)m * N + n, sum, N - n, n + 3 < N && (N & 3) == 0);
+                    });
                 }
             }
             turn = (turn + kStreamEpoch * FMX) % waves;
@@ -842,13 +846,15 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_basic_kernel(
         const int n = n0 + 4 * (l >> 4);
         if (m < M) {
             const float rs = ep.row_scale ? ep.row_scale[m] : 1.f;
+            by_output_width(ep, [&](auto half) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int nn = n + q < N ? n + q : N - 1;
-                s[q] = epilogue_value(ep, s[q], ep.bias ? ep.bias[nn] : 0, rs,
-                                      ep.col_scale ? ep.col_scale[nn] : 1.f);
-            }
-            store_out4(ep, Y, (size_t)m * N + n, s, N - n, n + 3 < N && (N & 3) == 0);
+                for (int q = 0; q < 4; ++q) {
+                    const int nn = n + q < N ? n + q : N - 1;
+                    s[q] = epilogue_value_of<half()>(ep, s[q], ep.bias ? ep.bias[nn] : 0, rs,
+                                                     ep.col_scale ? ep.col_scale[nn] : 1.f);
+                }
+                store_out4<half()>(Y, (size_t)m * N + n, s, N - n, n + 3 < N && (N & 3) == 0);
+            });
         }
     }
 }

@@ -119,15 +119,15 @@ int oracle_is_same(const int *a, const int *b, int count)
  * the 32 bits of ((float)v * row_scale[i]) * col_scale[j].  Null operands count as 0 / 1.
  * Compiled without floating-point contraction; the two products round separately. */
 /* float -> IEEE half, round to nearest even; beyond the largest half it is infinity, a NaN
- * becomes the quiet NaN 0x7e00 with the sign kept. */
+ * keeps its sign and the upper nine payload bits and becomes quiet. */
 unsigned oracle_f32_to_f16_bits(float f)
 {
     union { float f; uint32_t u; } v;
     v.f = f;
     const uint32_t sign = (v.u >> 16) & 0x8000u;
     const uint32_t x = v.u & 0x7fffffffu;
-    if (x > 0x7f800000u)
-        return sign | 0x7e00u;
+    if (x > 0x7f800000u) /* a NaN keeps its sign and upper payload bits and becomes quiet */
+        return sign | 0x7e00u | ((x >> 13) & 0x1ffu);
     if (x >= 0x47800000u) /* 65536 and up, infinity included */
         return sign | 0x7c00u;
     if (x >= 0x38800000u) { /* at least 2^-14: a normal half unless the rounding carries into infinity */

@@ -88,3 +88,24 @@ def check_half_width_outputs(xd, wd, want: np.ndarray, bias: np.ndarray, rs: np.
         got = y16.cpu().numpy().view(np.uint16)
         assert np.array_equal(got[:m * n].reshape(m, n), oracle.epilogue(want, bias, rs_small, cs, out=kind)), f"{kind} {kernel}"
         assert np.all(got[m * n:] == 0x7BAD), f"{kind} {kernel}: wrote past the output"
+
+
+def special_floats(seed: int) -> np.ndarray:
+    """Floats on which a conversion to half or bfloat16 is most likely to go wrong: every half
+    value, the midpoints between neighbouring halves and bfloat16s and the floats next to them,
+    the ends of both ranges, denormals, infinities, NaNs of both signs with several payloads,
+    and random bit patterns."""
+    rng = np.random.default_rng(seed)
+    h = np.arange(0x10000, dtype=np.uint16).view(np.float16).astype(np.float32)
+    hs = np.sort(np.unique(h[np.isfinite(h)]))
+    mid = ((hs[:-1].astype(np.float64) + hs[1:].astype(np.float64)) / 2).astype(np.float32)
+    near = np.concatenate([np.nextafter(mid, np.float32(np.inf)), np.nextafter(mid, np.float32(-np.inf))])
+    b = (np.arange(0x10000, dtype=np.uint32) << 16)
+    bf_ties = b | 0x8000
+    bf_near = np.concatenate([b | 0x7FFF, b | 0x8001, b | 0xFFFF, b | 0x0001])
+    edge = np.array([65504.0, 65519.99, 65520.0, 65520.01, 65536.0, 1e6, 3.4e38, np.inf, 2.0**-24, 2.0**-25,
+                     np.nextafter(np.float32(2.0**-25), np.float32(1)), 2.0**-26, 0.0], dtype=np.float32)
+    nans = np.array([0x7FC00000, 0xFFC00000, 0x7FC12345, 0xFFC54321, 0x7FE00000, 0x7FFFFFFF, 0xFFFFFFFF], dtype=np.uint32)
+    rnd = rng.integers(0, 2**32, size=100000, dtype=np.uint64).astype(np.uint32)
+    return np.concatenate([h, mid, near, bf_ties.view(np.float32), bf_near.view(np.float32), edge, -edge,
+                           nans.view(np.float32), rnd.view(np.float32)])

@@ -2,7 +2,7 @@
 // launches, 50 timed ones, every timed launch preceded by a cache-cleaning fill and bracketed
 // by its own event pair, median reported as 2*M*N*K / t in TOPS ("[PERF] ... TOPS").
 //
-//   benchmark [--kernel auto|simple|mfma|mfma128|mfma256|skinny|fp6] [--epilogue none|bias|f32]
+//   benchmark [--kernel auto|simple|mfma|mfma128|mfma256|skinny|fp6] [--epilogue none|bias|f32|f16|bf16]
 //             [--entry v0|v1|v2|v10|v11|v20|v21] [--iters I] [--warmup W] [--no-flush] MxNxK ...
 //
 // --entry times one of the reference's blocking linear_vN_launch entry points instead (each a
@@ -12,7 +12,8 @@
 // that step.
 //
 // --epilogue bias times int4linear_linear_s32 (bias add fused into the store), f32 times
-// int4linear_linear_f32 (bias, per-row and per-column scales, float output).
+// int4linear_linear_f32 (bias, per-row and per-column scales, float output), f16 / bf16 the
+// same with a half-width output.
 //
 // The reference cleans twice its L2 (benchmark.cu:77-91); an MI355X also has a 256 MiB
 // memory-side cache behind the eight L2s, so the fill here is 512 MiB.  Operand values are
@@ -76,7 +77,7 @@ int main(int argc, char **argv)
         }
     }
     const int kid = kernel_id(kernel);
-    if (kid < 0 || iters < 1 || (epilogue != "none" && epilogue != "bias" && epilogue != "f32")) {
+    if (kid < 0 || iters < 1 || (epilogue != "none" && epilogue != "bias" && epilogue != "f32" && epilogue != "f16" && epilogue != "bf16")) {
         std::fprintf(stderr, "bad --kernel, --epilogue or --iters\n");
         return 2;
     }
@@ -118,6 +119,12 @@ int main(int argc, char **argv)
             else if (epilogue == "f32")
                 st = int4linear_linear_f32(xd.p, wd.p, (const int *)bias.p, (const float *)rscale.p,
                                            (const float *)cscale.p, (float *)yd.p, m, n, k, kid, nullptr);
+            else if (epilogue == "f16")
+                st = int4linear_linear_f16(xd.p, wd.p, (const int *)bias.p, (const float *)rscale.p,
+                                           (const float *)cscale.p, yd.p, m, n, k, kid, nullptr);
+            else if (epilogue == "bf16")
+                st = int4linear_linear_bf16(xd.p, wd.p, (const int *)bias.p, (const float *)rscale.p,
+                                            (const float *)cscale.p, yd.p, m, n, k, kid, nullptr);
             else
                 st = int4linear_gemm_s4s4s32_ex(xd.p, wd.p, yd.p, m, n, k, kid, nullptr);
             if (st != INT4LINEAR_OK) {

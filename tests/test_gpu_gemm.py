@@ -236,6 +236,48 @@ def test_linear_with_epilogue(gpu, host_threads, m, n, k, kernels):
             assert np.array_equal(y16.cpu().numpy().view(np.uint16)[:m * n].reshape(m, n), plain_16[kind]), f"{kind} plain {kern}"
 
 
+@pytest.mark.parametrize("kernel", ["auto", "simple", "mfma", "fp6", "skinny"])
+def test_half_width_outputs_of_special_values(gpu, kernel):
+    """Every accumulator is 1 (one nonzero nibble per row), so output (i, j) is the conversion
+    of row_scale[i] * col_scale[j]: the hardware's float -> half and float -> bfloat16 against
+    the oracle's on halves, ties, range ends, denormals, infinities and quiet NaNs."""
+    import torch
+
+    import int4linear_amd as lib
+
+    v = helpers.special_floats(31)
+    snan = (v.view(np.uint32) & 0x7FC00000) == 0x7F800000
+    snan &= (v.view(np.uint32) & 0x003FFFFF) != 0
+    v = v[~snan]    # a signalling NaN is quieted by the multiplication: left to the quiet ones
+    rows = 16384 if kernel != "skinny" else 64
+    n, k = 16, 128
+    cs = np.array([1, 0.5, 2, 1, 0.75, 3, 1, 0.125, 1, 1, 1.5, 1, 4, 1, 1, 0.25], dtype=np.float32)
+    x = np.zeros((rows, k), dtype=np.int8)
+    x[:, 5] = 1
+    w = np.zeros((n, k), dtype=np.int8)
+    w[:, 5] = 1
+    xd = helpers.to_device_bytes(helpers.pack_bytes(x))
+    wd = helpers.to_device_bytes(helpers.pack_bytes(w))
+    ones = np.ones((rows, n), dtype=np.int32)
+    y = torch.zeros((rows, n), dtype=torch.int32, device="cuda:0")
+    lib.linear_s32(xd, wd, None, y, rows, n, k, kernel=kernel)
+    assert np.array_equal(y.cpu().numpy(), ones)
+    cd = torch.from_numpy(cs).to("cuda:0")
+    if kernel not in ("auto", "simple"):   # those go through all of them, the others through a sample with the range ends and NaNs
+        pick = np.random.default_rng(32).choice(len(v), max(4 * rows, 4096) - 40, replace=False)
+        v = np.concatenate([v[pick], v[len(v) - 100040:len(v) - 100000]])
+    for first in range(0, len(v), rows):
+        rs = np.resize(v[first:first + rows], rows).astype(np.float32)
+        rd = torch.from_numpy(rs).to("cuda:0")
+        for kind, fn in (("f16", lib.linear_f16), ("bf16", lib.linear_bf16)):
+            y16 = torch.zeros((rows, n), dtype=torch.int16, device="cuda:0")
+            fn(xd, wd, None, rd, cd, y16, rows, n, k, kernel=kernel)
+            got = y16.cpu().numpy().view(np.uint16)
+            want = oracle.epilogue(ones, None, rs, cs, out=kind)
+            bad = np.argwhere(got != want)
+            assert bad.size == 0, (kind, kernel, first, bad[:3], [hex(int(rs.view(np.uint32)[i])) for i, _ in bad[:3]])
+
+
 def test_internal_workspace_shared_between_streams(gpu, host_threads):
     """Calls that use the FP6 workspace from alternating streams, without any host
     synchronisation in between: the library orders them itself."""

@@ -159,6 +159,12 @@ def test_half_conversion_against_numpy():
         want = v.astype(np.float16).view(np.uint16)
     got = oracle.convert_f32(v, "f16")
     assert np.array_equal(got, want), np.flatnonzero(got != want)[:5]
+    # quiet NaNs: sign and upper payload kept (numpy's rule as well)
+    q = helpers.special_floats(24)
+    q = q[np.isnan(q) & ((q.view(np.uint32) & 0x00400000) != 0)]
+    assert len(q) > 100
+    assert np.array_equal(oracle.convert_f32(q, "f16"), q.astype(np.float16).view(np.uint16))
+    assert oracle.convert_f32(np.array([0x7F800001], np.uint32).view(np.float32), "f16")[0] == 0x7E00  # a signalling NaN comes out quiet
 
 
 def test_bfloat16_conversion_against_torch():
@@ -175,6 +181,10 @@ def test_bfloat16_conversion_against_torch():
     assert np.array_equal(got, want), np.flatnonzero(got != want)[:5]
     exact = (np.arange(0x7F80, dtype=np.uint32) << 16).view(np.float32)   # every finite bfloat16 value
     assert np.array_equal(oracle.convert_f32(exact, "bf16"), np.arange(0x7F80, dtype=np.uint16))
+    # NaNs: the upper half with the quiet bit set
+    q = helpers.special_floats(25)
+    q = q[np.isnan(q)]
+    assert np.array_equal(oracle.convert_f32(q, "bf16"), ((q.view(np.uint32) >> 16) | 0x40).astype(np.uint16))
     assert oracle.convert_f32(np.array([1.00390625], np.float32), "bf16")[0] == 0x3F80       # 1 + 2^-8 ties down to even
     assert oracle.convert_f32(np.array([1.01171875], np.float32), "bf16")[0] == 0x3F82       # 1 + 3 * 2^-8 ties up to even
 
