@@ -56,17 +56,15 @@ __device__ __forceinline__ int epilogue_value16(const Epilogue &ep, int acc, int
     return (int)__builtin_bit_cast(unsigned short, (__bf16)t);
 }
 
-__device__ __forceinline__ bool out_is_half_width(const Epilogue &ep);
+__device__ __forceinline__ bool out_is_half_width(const Epilogue &ep) { return ep.out >= kOutF16; }
 
 // Either of them, by the kind of output.
 __device__ __forceinline__ int epilogue_value(const Epilogue &ep, int acc, int bias_j, float row_scale_i,
                                               float col_scale_j)
 {
-    return ep.out >= kOutF16 ? epilogue_value16(ep, acc, bias_j, row_scale_i, col_scale_j)
-                             : epilogue_value32(ep, acc, bias_j, row_scale_i, col_scale_j);
+    return out_is_half_width(ep) ? epilogue_value16(ep, acc, bias_j, row_scale_i, col_scale_j)
+                                 : epilogue_value32(ep, acc, bias_j, row_scale_i, col_scale_j);
 }
-
-__device__ __forceinline__ bool out_is_half_width(const Epilogue &ep) { return ep.out >= kOutF16; }
 
 // Element `index` of the output array, whichever its width.
 __device__ __forceinline__ void store_out(const Epilogue &ep, void *c, size_t index, int bits)
