@@ -28,7 +28,10 @@
  *                        oracle_f32_to_bf16_bits: one more rounding to nearest even) are
  *                        pinned against numpy's float16 conversion over every float16 value,
  *                        every halfway point between neighbours and random floats, and
- *                        against torch's bfloat16 conversion likewise.
+ *                        against torch's bfloat16 conversion likewise; quiet NaNs (sign
+ *                        and upper payload bits kept) against numpy for the half and
+ *                        against the closed form (upper 16 bits, quiet bit set) for
+ *                        bfloat16.
  */
 #include <stddef.h>
 #include <stdint.h>
@@ -114,10 +117,6 @@ int oracle_is_same(const int *a, const int *b, int count)
     return 1;
 }
 
-/* The epilogue of int4linear_linear_s32 / _f32, applied in place to a finished int32
- * product y (m x n): v = y[i][j] + bias[j] (two's-complement wrap), and for f32 != 0
- * the 32 bits of ((float)v * row_scale[i]) * col_scale[j].  Null operands count as 0 / 1.
- * Compiled without floating-point contraction; the two products round separately. */
 /* float -> IEEE half, round to nearest even; beyond the largest half it is infinity, a NaN
  * keeps its sign and the upper nine payload bits and becomes quiet. */
 unsigned oracle_f32_to_f16_bits(float f)
@@ -168,21 +167,26 @@ void oracle_convert_f32(const float *src, unsigned short *dst, size_t n, int kin
         dst[i] = (unsigned short)(kind == 2 ? oracle_f32_to_f16_bits(src[i]) : oracle_f32_to_bf16_bits(src[i]));
 }
 
-/* `out`: 0 int32, 1 float32 (its bits), 2 half, 3 bfloat16 (16 bits in the low half of the int). */
+/* The epilogue of int4linear_linear_s32 / _f32 / _f16 / _bf16, applied in place to a finished
+ * int32 product y (m x n): v = y[i][j] + bias[j] (two's-complement wrap), and for out != 0
+ * t = ((float)v * row_scale[i]) * col_scale[j].  Null operands count as 0 / 1.
+ * Compiled without floating-point contraction; the two products round separately.
+ * `out`: 0 int32 (v), 1 float32 (the bits of t), 2 half, 3 bfloat16 (t rounded once more; the
+ * 16 bits in the low half of the int). */
 void oracle_epilogue(int *y, int m, int n, const int *bias, const float *row_scale,
-                     const float *col_scale, int f32)
+                     const float *col_scale, int out)
 {
     for (int i = 0; i < m; ++i) {
         const float rs = row_scale ? row_scale[i] : 1.0f;
         for (int j = 0; j < n; ++j) {
             const uint32_t sum = (uint32_t)y[(size_t)i * n + j] + (uint32_t)(bias ? bias[j] : 0);
             int v = (int)sum;
-            if (f32) {
+            if (out) {
                 volatile float a = (float)v * rs;  /* volatile: no fused or reassociated product */
                 const float f = a * (col_scale ? col_scale[j] : 1.0f);
                 union { float f; int i; } u;
                 u.f = f;
-                v = f32 == 2 ? (int)oracle_f32_to_f16_bits(f) : f32 == 3 ? (int)oracle_f32_to_bf16_bits(f) : u.i;
+                v = out == 2 ? (int)oracle_f32_to_f16_bits(f) : out == 3 ? (int)oracle_f32_to_bf16_bits(f) : u.i;
             }
             y[(size_t)i * n + j] = v;
         }
