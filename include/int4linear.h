@@ -16,10 +16,20 @@
  * All pointers named *_d are device pointers owned by the caller.  The only device
  * memory the library itself allocates is one workspace per device (see
  * int4linear_workspace_bytes), which holds the FP6 kernel's converted operands and the
- * partial sums of either MFMA kernel's split-K form: created on first need, grown when a
- * larger problem arrives, never larger than the workspace limit, freed by
- * int4linear_release_workspace or at process exit.  With the limit set to 0 no entry
- * point allocates anything.  A call whose stream is being captured into a HIP graph never
+ * partial sums of the split-K forms: created on first need, grown when a larger problem
+ * arrives, never larger than the workspace limit, freed by int4linear_release_workspace;
+ * a process that never calls that keeps it until it ends (the library installs no exit
+ * handler).  With the limit set to 0 no entry point allocates anything.  Besides that the
+ * library's device image holds the fixed scratch array of int4linear_gemm_s4s4s32_static
+ * (INT4LINEAR_STATIC_SCRATCH_BYTES, 128 MiB of device memory on every device a process
+ * initialises the library on, whether or not that entry point is ever called) and 64 KiB
+ * of counters.
+ *
+ * HIP graphs: the first call on a device sets the library up (device queries, kernel
+ * attributes, the address of the scratch array), which must not happen inside a capture:
+ * call int4linear_init(), or any other entry point, on the device before the capture
+ * begins; a first call that arrives while its stream is capturing returns
+ * INT4LINEAR_ERR_NOT_INITIALISED.  A call whose stream is being captured into a HIP graph never
  * touches that workspace either: under automatic dispatch it runs the kernels that need
  * none, and an explicit INT4LINEAR_KERNEL_FP6 request returns INT4LINEAR_ERR_UNSUPPORTED
  * (graphs that want the FP6 kernel use int4linear_gemm_fp6_converted on their own buffers,
@@ -43,8 +53,19 @@ enum {
     INT4LINEAR_ERR_HIP = 4,         /* a HIP runtime call failed (see last_hip_error)    */
     INT4LINEAR_ERR_UNSUPPORTED = 5, /* the requested kernel cannot run this shape        */
     INT4LINEAR_ERR_NO_DEVICE = 6,   /* no gfx950 device is visible                       */
-    INT4LINEAR_ERR_SCRATCH = 7      /* int4linear_gemm_s4s4s32_static: the shape needs more
-                                       than INT4LINEAR_STATIC_SCRATCH_BYTES of scratch   */
+    INT4LINEAR_ERR_SCRATCH = 7,     /* int4linear_gemm_s4s4s32_static: the only fast kernel
+                                       for the shape needs more scratch memory than
+                                       INT4LINEAR_STATIC_SCRATCH_BYTES                   */
+    INT4LINEAR_ERR_NOT_INITIALISED = 8 /* first call on this device while its stream is being
+                                       captured: call int4linear_init() before capturing */
+};
+
+/* Element type of the output of int4linear_linear_fp6_converted. */
+enum {
+    INT4LINEAR_OUT_S32 = 0,  /* int32: sum + bias                                         */
+    INT4LINEAR_OUT_F32 = 1,  /* float: ((float)(sum + bias) * row_scale) * col_scale      */
+    INT4LINEAR_OUT_F16 = 2,  /* the float value rounded to IEEE half                      */
+    INT4LINEAR_OUT_BF16 = 3  /* the float value rounded to bfloat16                       */
 };
 
 /* Kernel selector for int4linear_gemm_s4s4s32_ex. */
@@ -63,9 +84,10 @@ enum {
 };
 
 /* One-time set-up for the current HIP device (queries the CU count, raises the
- * dynamic-LDS limit of the kernels).  Called implicitly by the other entry points;
- * idempotent and thread-safe.  Replaces the per-call cudaFuncSetAttribute of
- * kernels/linear_v21.cu:14-18. */
+ * dynamic-LDS limit of the kernels, takes the addresses of the scratch arrays).  Called
+ * implicitly by the other entry points, except while their stream is being captured (see
+ * above); idempotent and thread-safe; a failed set-up is tried again by the next call.
+ * Replaces the per-call cudaFuncSetAttribute of kernels/linear_v21.cu:14-18. */
 int int4linear_init(void);
 
 /* The GEMM.  Asynchronous: work is enqueued on `stream` (a hipStream_t, NULL = the
@@ -80,15 +102,17 @@ int int4linear_gemm_s4s4s32(const void *a_packed_d, const void *b_packed_d, void
  * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart
  * in the reference (whose launcher needs no scratch memory, kernels/linear_v21.cu:9-49).
  * Same arguments, same result, same choice of kernel as int4linear_gemm_s4s4s32 makes with
- * an unlimited workspace, but where that entry point would use its allocated workspace (the
+ * a workspace limit of the array's size, but where that entry point would use its allocated workspace (the
  * FP6 kernel's converted operands, the partial sums of the split-K forms) this one uses a
  * fixed array of INT4LINEAR_STATIC_SCRATCH_BYTES that is part of the library's device image:
  * every device the library is initialised on holds one copy until the process ends.  The
  * call allocates and frees nothing, records no events and takes no locks.  A shape whose
- * kernel would need more scratch than the array holds is refused with
- * INT4LINEAR_ERR_SCRATCH before anything is enqueued (at M = N = K the FP6 form fits up to
- * 9216; use int4linear_gemm_s4s4s32_ex with INT4LINEAR_KERNEL_MFMA for larger problems, it
- * needs no scratch at all).  All calls on one device share the one array and nothing orders
+ * kernel would need more scratch than the array holds (at M = N = K the FP6 form fits up to
+ * 9216) runs on the kernels that need none, as it does under graph capture through the
+ * ordinary entry point; only when that would leave a large problem to the scalar kernel (K
+ * not a multiple of 128, which among the fast kernels only the FP6 one takes) is the call
+ * refused with INT4LINEAR_ERR_SCRATCH before anything is enqueued.  Set the device up
+ * (int4linear_init) before capturing.  All calls on one device share the one array and nothing orders
  * them: calls whose execution may overlap on a device (different streams, graphs replayed
  * concurrently) race on it; calls on one stream are ordered by the stream. */
 #define INT4LINEAR_STATIC_SCRATCH_BYTES (128u << 20)
@@ -143,11 +167,22 @@ int int4linear_unpack_s4_to_s32(const int *src_d, int *dst_d, int m, int n, void
  *   int4linear_fp6_convert        packed s4 (rows x k/2 bytes) -> converted form;
  *                                 converted_d must be 256-byte aligned;
  *   int4linear_gemm_fp6_converted C = A * B^T from two converted operands.
- * The converted form is opaque and specific to this library version. */
+ *   int4linear_linear_fp6_converted the same product with the epilogue of the
+ *                                 int4linear_linear_* entry points fused into the store
+ *                                 (bias_d, row_scale_d, col_scale_d may each be NULL; out_type
+ *                                 is an INT4LINEAR_OUT_* value and y_d an m x n array of that
+ *                                 type; INT4LINEAR_OUT_S32 takes a bias only).  The
+ *                                 README's bias add (README.md:72) on the path a layer
+ *                                 with static weights uses.
+ * The converted form is opaque and specific to this library version.  Neither GEMM entry
+ * point allocates or touches the library's workspace: both may be captured into a graph. */
 size_t int4linear_fp6_operand_bytes(int rows, int k);
 int int4linear_fp6_convert(const void *packed_d, void *converted_d, int rows, int k, void *stream);
 int int4linear_gemm_fp6_converted(const void *a_conv_d, const void *b_conv_d, void *c_d,
                                   int m, int n, int k, void *stream);
+int int4linear_linear_fp6_converted(const void *x_conv_d, const void *w_conv_d, const int *bias_d,
+                                    const float *row_scale_d, const float *col_scale_d, void *y_d,
+                                    int out_type, int m, int n, int k, void *stream);
 
 /* Bytes of internal workspace INT4LINEAR_KERNEL_AUTO would use for a shape on the current
  * device (0 when the chosen kernel needs none).  Sets the device up if that has not

@@ -15,6 +15,7 @@ from .api import (  # noqa: F401
     linear_bf16,
     linear_f16,
     linear_f32,
+    linear_fp6_converted,
     linear_s32,
     linear_v0_launch,
     linear_v1_launch,

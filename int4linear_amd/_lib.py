@@ -33,6 +33,8 @@ C_ABI = [
     ("int4linear_fp6_operand_bytes", c_size_t, [c_int, c_int]),
     ("int4linear_fp6_convert", c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
     ("int4linear_gemm_fp6_converted", c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    ("int4linear_linear_fp6_converted", c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                                                c_int, c_int, c_int, c_void_p]),
     ("int4linear_workspace_bytes", c_size_t, [c_int, c_int, c_int]),
     ("int4linear_set_workspace_limit", None, [c_size_t]),
     ("int4linear_release_workspace", c_int, []),

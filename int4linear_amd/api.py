@@ -130,6 +130,21 @@ def gemm_fp6_converted(a_conv_d, b_conv_d, c_d, m: int, n: int, k: int, *, strea
                                                  ctypes.c_void_p(stream)))
 
 
+OUT_TYPES = {"s32": 0, "f32": 1, "f16": 2, "bf16": 3}  # INT4LINEAR_OUT_*
+
+
+def linear_fp6_converted(x_conv_d, w_conv_d, bias_d, row_scale_d, col_scale_d, y_d, out_type: str, m: int, n: int,
+                         k: int, *, stream: int | None = None) -> None:
+    """gemm_fp6_converted with the epilogue of linear_s32 / linear_f32 / linear_f16 / linear_bf16
+    (out_type "s32", "f32", "f16" or "bf16"); bias_d and the scales may each be None."""
+    lib = _lib.load()
+    if stream is None:
+        stream = _current_stream()
+    _lib.check(lib.int4linear_linear_fp6_converted(_ptr(x_conv_d), _ptr(w_conv_d), _ptr(bias_d), _ptr(row_scale_d),
+                                                   _ptr(col_scale_d), _ptr(y_d), OUT_TYPES[out_type], m, n, k,
+                                                   ctypes.c_void_p(stream)))
+
+
 def workspace_bytes(m: int, n: int, k: int) -> int:
     """Internal workspace the automatic dispatch would use for this shape."""
     return int(_lib.load().int4linear_workspace_bytes(m, n, k))

@@ -36,7 +36,9 @@ HIP_FLAGS = [
 # of its kernel arguments are a memory round trip in front of its first instruction that does
 # anything: there the first 14 dwords of the arguments arrive preloaded in scalar registers.
 # (The compiler keeps a prologue that loads them the ordinary way, which firmware without the
-# feature runs instead.)
+# feature runs instead.)  The option is internal to LLVM: build_library() tries it on an empty
+# kernel first and drops it if this hipcc does not take it (the kernels then load their
+# arguments the ordinary way, a few tenths of a microsecond per launch).
 EXTRA_HIP_FLAGS = {
     "kernels_skinny.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=14"],
 }
@@ -47,6 +49,22 @@ def _hipcc() -> str:
     if not os.path.exists(exe):
         raise RuntimeError("hipcc not found; ROCm is required to build int4linear_amd")
     return exe
+
+
+def _accepted_flags(hipcc: str, flags: list[str]) -> list[str]:
+    """`flags` if this hipcc compiles an empty device function with them, else none of them:
+    options passed to LLVM with -mllvm are internal and may be gone in another release, and a
+    missing one must cost its tuning, not the build."""
+    import tempfile
+
+    with tempfile.TemporaryDirectory() as tmp:
+        src = Path(tmp) / "probe.hip"
+        src.write_text("__global__ void probe(int *p) { *p = 0; }\n")
+        cmd = [hipcc, "--offload-arch=gfx950", "--cuda-device-only", *flags, "-c", str(src), "-o", str(Path(tmp) / "probe.o")]
+        ok = subprocess.run(cmd, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL).returncode == 0
+    if not ok:
+        sys.stderr.write("int4linear_amd.build: hipcc rejects " + " ".join(flags) + "; building without\n")
+    return flags if ok else []
 
 
 def _run(cmd: list[str]) -> None:
@@ -81,7 +99,8 @@ def build_library(verbose: bool = False, save_temps: bool = False) -> Path:
     jobs = []
     for src in HIP_SOURCES:
         obj = OBJ_DIR / (src + ".o")
-        cmd = [hipcc, *HIP_FLAGS, *EXTRA_HIP_FLAGS.get(src, []), "-c", str(CSRC / src), "-o", str(obj)]
+        extra = _accepted_flags(hipcc, EXTRA_HIP_FLAGS[src]) if src in EXTRA_HIP_FLAGS else []
+        cmd = [hipcc, *HIP_FLAGS, *extra, "-c", str(CSRC / src), "-o", str(obj)]
         if save_temps:
             cmd.insert(1, "-save-temps=obj")
         jobs.append((cmd, obj))

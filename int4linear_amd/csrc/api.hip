@@ -21,13 +21,21 @@ constexpr int kMaxDevices = 64;
 // uses PerDevice::scratch.
 constexpr size_t kStaticScratchBytes = (size_t)INT4LINEAR_STATIC_SCRATCH_BYTES;
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+// Arrival counters of the weight-streaming kernel's split over K (kernels.h): two sets, the
+// first for calls that keep their partial sums in the internal workspace, the second for
+// int4linear_gemm_s4s4s32_static.  Zero when the library is loaded; every launch leaves them
+// zero again.
+static __device__ __align__(256) unsigned arrivals[2][kSkinnyArrivalWords];
 
 struct PerDevice {
-    std::once_flag once;
-    hipError_t init_error = hipSuccess;
-    int status = INT4LINEAR_OK;
+    // Set-up happens once per device, under init_mutex; `ready` is set only when it has
+    // succeeded, so a failure (a transient one included) is reported to the caller that
+    // met it and tried again by the next call.
+    std::mutex init_mutex;
+    std::atomic<bool> ready{false};
     DeviceInfo info;
     void *scratch = nullptr;  // this device's copy of `scratch` (kStaticScratchBytes bytes)
+    unsigned *arrivals = nullptr;  // this device's copy of `arrivals`
     // Workspace of the FP6 path: grown on demand up to g_workspace_limit, kept until
     // int4linear_release_workspace() or process exit.  `ws_event` marks the end of the
     // last GEMM that used it, so a call on another stream can wait for it.
@@ -50,8 +58,45 @@ int fail_hip(hipError_t e)
     return INT4LINEAR_ERR_HIP;
 }
 
-// Set-up for the device that is current on the calling thread; returns its record.
-int ensure_init(PerDevice **out)
+// True while `stream` records into a graph.  Allocating, freeing and recording events on
+// other streams are all off limits then, and so is baking the internal workspace's address
+// into a graph that may outlive it.  A query that fails counts as capturing.
+bool stream_is_capturing(hipStream_t stream)
+{
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
+        (void)hipGetLastError();
+        return true;
+    }
+    return status != hipStreamCaptureStatusNone;
+}
+
+hipError_t set_up_device(PerDevice &pd, int dev)
+{
+    hipDeviceProp_t prop;
+    hipError_t err = hipGetDeviceProperties(&prop, dev);
+    if (err != hipSuccess)
+        return err;
+    pd.info.cu_count = prop.multiProcessorCount;
+    pd.info.lds_per_cu = (int)prop.maxSharedMemoryPerMultiProcessor;
+    err = mfma_init(pd.info);
+    if (err == hipSuccess)
+        err = fp6_init(pd.info);
+    if (err == hipSuccess)
+        err = skinny_init(pd.info);
+    if (err == hipSuccess)  // `dev` is current here: the addresses are this device's copies
+        err = hipGetSymbolAddress((void **)&pd.scratch, HIP_SYMBOL(scratch));
+    if (err == hipSuccess)
+        err = hipGetSymbolAddress((void **)&pd.arrivals, HIP_SYMBOL(arrivals));
+    return err;
+}
+
+// Set-up for the device that is current on the calling thread; returns its record.  Set-up
+// queries the device, raises the dynamic-LDS limit of some 250 kernels and takes the address
+// of the scratch arrays (which loads the device image): none of that belongs inside a graph
+// capture, so a first call that arrives with `work_stream` capturing is refused
+// (`for_work`: the call is about to enqueue work on work_stream).
+int ensure_init(PerDevice **out, bool for_work = false, hipStream_t work_stream = nullptr)
 {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
@@ -62,31 +107,18 @@ int ensure_init(PerDevice **out)
     if (dev < 0 || dev >= kMaxDevices)
         return INT4LINEAR_ERR_NO_DEVICE;
     PerDevice &pd = g_devices[dev];
-    std::call_once(pd.once, [&pd, dev]() {
-        hipDeviceProp_t prop;
-        hipError_t err = hipGetDeviceProperties(&prop, dev);
-        if (err != hipSuccess) {
-            pd.init_error = err;
-            pd.status = INT4LINEAR_ERR_HIP;
-            return;
+    if (!pd.ready.load(std::memory_order_acquire)) {
+        if (for_work && stream_is_capturing(work_stream))
+            return INT4LINEAR_ERR_NOT_INITIALISED;
+        std::lock_guard<std::mutex> lock(pd.init_mutex);
+        if (!pd.ready.load(std::memory_order_relaxed)) {
+            e = set_up_device(pd, dev);
+            if (e != hipSuccess) {
+                (void)hipGetLastError();
+                return fail_hip(e);
+            }
+            pd.ready.store(true, std::memory_order_release);
         }
-        pd.info.cu_count = prop.multiProcessorCount;
-        pd.info.lds_per_cu = (int)prop.maxSharedMemoryPerMultiProcessor;
-        err = mfma_init(pd.info);
-        if (err == hipSuccess)
-            err = fp6_init(pd.info);
-        if (err == hipSuccess)
-            err = skinny_init(pd.info);
-        if (err == hipSuccess)  // `dev` is current here: the address is this device's copy
-            err = hipGetSymbolAddress((void **)&pd.scratch, HIP_SYMBOL(scratch));
-        if (err != hipSuccess) {
-            pd.init_error = err;
-            pd.status = INT4LINEAR_ERR_HIP;
-        }
-    });
-    if (pd.status != INT4LINEAR_OK) {
-        t_last_hip_error = (int)pd.init_error;
-        return pd.status;
     }
     if (out)
         *out = &pd;
@@ -151,19 +183,6 @@ enum class Workspace {
     None       // none: only kernels that need no workspace
 };
 
-// True while `stream` records into a graph.  Allocating, freeing and recording events on
-// other streams are all off limits then, and so is baking the internal workspace's address
-// into a graph that may outlive it.  A query that fails counts as capturing.
-bool stream_is_capturing(hipStream_t stream)
-{
-    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
-        (void)hipGetLastError();
-        return true;
-    }
-    return status != hipStreamCaptureStatusNone;
-}
-
 // Hands out the device's internal workspace with at least `need` bytes for work about to be
 // enqueued on `stream` (the caller holds pd->ws_mutex until that work is enqueued).  Calls
 // on one stream are ordered by the stream; a call on a different stream than the previous
@@ -218,9 +237,9 @@ int acquire_workspace(PerDevice *pd, size_t need, hipStream_t stream, void **out
 }
 
 // The FP6 path: converted operands (and split-K slabs) in the internal workspace or in the
-// static scratch array.
+// static scratch array.  `capturing`: the stream records into a graph (Internal only).
 int run_fp6(PerDevice *pd, const void *a, const void *b, void *c, int m, int n, int k,
-            const Epilogue &ep, Workspace source, hipStream_t stream)
+            const Epilogue &ep, Workspace source, bool capturing, hipStream_t stream)
 {
     const size_t need = fp6_workspace_bytes(m, n, k, pd->info);
     hipError_t e;
@@ -229,7 +248,7 @@ int run_fp6(PerDevice *pd, const void *a, const void *b, void *c, int m, int n, 
             return INT4LINEAR_ERR_SCRATCH;
         e = launch_fp6(a, b, c, m, n, k, pd->scratch, ep, pd->info, stream);
     } else {
-        if (source == Workspace::None || stream_is_capturing(stream))
+        if (source == Workspace::None || capturing)
             return INT4LINEAR_ERR_UNSUPPORTED;
         std::lock_guard<std::mutex> lock(pd->ws_mutex);
         void *ws = nullptr;
@@ -244,24 +263,44 @@ int run_fp6(PerDevice *pd, const void *a, const void *b, void *c, int m, int n, 
 // The int8 kernel under automatic dispatch: split over K when that helps and the workspace
 // for the partial sums can be had, otherwise the plain kernel.
 int run_mfma_auto(PerDevice *pd, const void *a, const void *b, void *c, int m, int n, int k,
-                  const Epilogue &ep, Workspace source, hipStream_t stream)
+                  const Epilogue &ep, Workspace source, bool capturing, hipStream_t stream)
 {
     const size_t need = mfma_workspace_bytes(m, n, k, pd->info);
     hipError_t e;
-    if (need == 0) {
+    if (need == 0 || source == Workspace::None || capturing ||
+        (source == Workspace::Static && need > kStaticScratchBytes)) {
         e = launch_mfma(a, b, c, m, n, k, ep, pd->info, stream);
     } else if (source == Workspace::Static) {
-        if (need > kStaticScratchBytes)
-            return INT4LINEAR_ERR_SCRATCH;
         e = launch_mfma_splitk(a, b, c, m, n, k, pd->scratch, ep, pd->info, stream);
-    } else if (source == Workspace::None || stream_is_capturing(stream)) {
-        e = launch_mfma(a, b, c, m, n, k, ep, pd->info, stream);
     } else {
         std::lock_guard<std::mutex> lock(pd->ws_mutex);
         void *ws = nullptr;
         if (acquire_workspace(pd, need, stream, &ws) != INT4LINEAR_OK)
             ws = nullptr;  // no workspace: the unsplit kernel
         e = launch_mfma_splitk(a, b, c, m, n, k, ws, ep, pd->info, stream);
+    }
+    return e == hipSuccess ? INT4LINEAR_OK : fail_hip(e);
+}
+
+// The weight-streaming kernel under automatic dispatch: the shapes it splits over K across
+// workgroups keep their partial sums in the workspace; without one they run unsplit.
+int run_skinny_auto(PerDevice *pd, const void *a, const void *b, void *c, int m, int n, int k,
+                    const Epilogue &ep, Workspace source, bool capturing, hipStream_t stream)
+{
+    const size_t need = skinny_workspace_bytes(m, n, k, pd->info);
+    hipError_t e;
+    if (need == 0 || source == Workspace::None || capturing ||
+        (source == Workspace::Static && need > kStaticScratchBytes)) {
+        e = launch_skinny(a, b, c, m, n, k, ep, pd->info, stream);
+    } else if (source == Workspace::Static) {
+        e = launch_skinny_ksplit(a, b, c, m, n, k, pd->scratch, pd->arrivals + kSkinnyArrivalWords, ep, pd->info, stream);
+    } else {
+        std::lock_guard<std::mutex> lock(pd->ws_mutex);
+        void *ws = nullptr;
+        if (acquire_workspace(pd, need, stream, &ws) == INT4LINEAR_OK)
+            e = launch_skinny_ksplit(a, b, c, m, n, k, ws, pd->arrivals, ep, pd->info, stream);
+        else
+            e = launch_skinny(a, b, c, m, n, k, ep, pd->info, stream);
     }
     return e == hipSuccess ? INT4LINEAR_OK : fail_hip(e);
 }
@@ -282,11 +321,11 @@ int gemm_impl(const void *a, const void *b, void *c, int m, int n, int k, int ke
     if (!aligned16(c) || (k > 0 && (!aligned16(a) || !aligned16(b))))
         return INT4LINEAR_ERR_ALIGN;
 
+    hipStream_t stream = (hipStream_t)stream_v;
     PerDevice *pd = nullptr;
-    int st = ensure_init(&pd);
+    int st = ensure_init(&pd, true, stream);
     if (st != INT4LINEAR_OK)
         return st;
-    hipStream_t stream = (hipStream_t)stream_v;
 
     const bool plain = !ep.bias && !ep.row_scale && !ep.col_scale && !ep.out;
     if (k == 0 && plain) {
@@ -299,20 +338,35 @@ int gemm_impl(const void *a, const void *b, void *c, int m, int n, int k, int ke
     }
 
     const bool automatic = kernel == INT4LINEAR_KERNEL_AUTO;
+    bool capturing = false;
     if (automatic) {
-        // The static scratch entry chooses as if memory were no object and then refuses what
-        // does not fit its array; a stream under capture gets the kernels without workspace.
-        size_t limit = g_workspace_limit.load();
-        if (source == Workspace::Static)
-            limit = SIZE_MAX;
-        else if (limit > 0 && stream_is_capturing(stream))
-            limit = 0;
+        const size_t limit = source == Workspace::Static ? kStaticScratchBytes : g_workspace_limit.load();
         kernel = pick_kernel(m, n, k, pd->info, limit);
+        // A stream under capture gets the kernels that need no workspace.  Whether it is one
+        // is asked only when the chosen kernel would touch the internal workspace or its
+        // ordering between streams: decode calls with up to 16 rows, a few microseconds
+        // long, never pay for the query.
+        if (source == Workspace::Internal &&
+            (kernel == INT4LINEAR_KERNEL_FP6 ||
+             (kernel == INT4LINEAR_KERNEL_MFMA && limit > 0 && mfma_workspace_bytes(m, n, k, pd->info) > 0) ||
+             (kernel == INT4LINEAR_KERNEL_SKINNY && limit > 0 && skinny_workspace_bytes(m, n, k, pd->info) > 0))) {
+            capturing = stream_is_capturing(stream);
+            if (capturing)
+                kernel = pick_kernel(m, n, k, pd->info, 0);
+        }
+        // The static entry point falls back to the kernels without scratch memory when the
+        // array is too small; it refuses only what would then be left to the scalar kernel
+        // although a fast kernel exists for it (ragged K beyond the array's size).
+        if (source == Workspace::Static && kernel == INT4LINEAR_KERNEL_SIMPLE &&
+            pick_kernel(m, n, k, pd->info, SIZE_MAX) != INT4LINEAR_KERNEL_SIMPLE)
+            return INT4LINEAR_ERR_SCRATCH;
+    } else if (kernel == INT4LINEAR_KERNEL_FP6 && source == Workspace::Internal) {
+        capturing = stream_is_capturing(stream);
     }
     if (kernel == INT4LINEAR_KERNEL_FP6) {
         if (!fp6_supports(m, n, k))
             return INT4LINEAR_ERR_UNSUPPORTED;
-        const int st6 = run_fp6(pd, a, b, c, m, n, k, ep, source, stream);
+        const int st6 = run_fp6(pd, a, b, c, m, n, k, ep, source, capturing, stream);
         // Under automatic dispatch a workspace that cannot be had falls back to a kernel
         // that needs none.
         if (st6 == INT4LINEAR_OK || !automatic || source == Workspace::Static)
@@ -329,7 +383,7 @@ int gemm_impl(const void *a, const void *b, void *c, int m, int n, int k, int ke
         if (!mfma_supports(m, n, k))
             return INT4LINEAR_ERR_UNSUPPORTED;
         if (automatic)
-            return run_mfma_auto(pd, a, b, c, m, n, k, ep, source, stream);
+            return run_mfma_auto(pd, a, b, c, m, n, k, ep, source, capturing, stream);
         e = launch_mfma(a, b, c, m, n, k, ep, pd->info, stream);
         break;
     case INT4LINEAR_KERNEL_MFMA_128:
@@ -342,6 +396,8 @@ int gemm_impl(const void *a, const void *b, void *c, int m, int n, int k, int ke
     case INT4LINEAR_KERNEL_SKINNY:
         if (!skinny_supports(m, n, k))
             return INT4LINEAR_ERR_UNSUPPORTED;
+        if (automatic)
+            return run_skinny_auto(pd, a, b, c, m, n, k, ep, source, capturing, stream);
         e = launch_skinny(a, b, c, m, n, k, ep, pd->info, stream);
         break;
     default:
@@ -442,7 +498,7 @@ int int4linear_pack_s32_to_s4(const int *src_d, int *dst_d, int m, int n, void *
         return INT4LINEAR_OK;
     if (!src_d || !dst_d)
         return INT4LINEAR_ERR_NULL;
-    int st = ensure_init(nullptr);
+    int st = ensure_init(nullptr, true, (hipStream_t)stream);
     if (st != INT4LINEAR_OK)
         return st;
     hipError_t e = launch_pack(src_d, dst_d, m, n, (hipStream_t)stream);
@@ -457,7 +513,7 @@ int int4linear_unpack_s4_to_s32(const int *src_d, int *dst_d, int m, int n, void
         return INT4LINEAR_OK;
     if (!src_d || !dst_d)
         return INT4LINEAR_ERR_NULL;
-    int st = ensure_init(nullptr);
+    int st = ensure_init(nullptr, true, (hipStream_t)stream);
     if (st != INT4LINEAR_OK)
         return st;
     hipError_t e = launch_unpack(src_d, dst_d, m, n, (hipStream_t)stream);
@@ -483,15 +539,19 @@ int int4linear_fp6_convert(const void *packed_d, void *converted_d, int rows, in
         return INT4LINEAR_ERR_NULL;
     if (!aligned16(packed_d) || ((uintptr_t)converted_d & 255) != 0)
         return INT4LINEAR_ERR_ALIGN;
-    int st = ensure_init(nullptr);
+    int st = ensure_init(nullptr, true, (hipStream_t)stream);
     if (st != INT4LINEAR_OK)
         return st;
     hipError_t e = launch_fp6_convert(packed_d, converted_d, rows, k, (hipStream_t)stream);
     return e == hipSuccess ? INT4LINEAR_OK : fail_hip(e);
 }
 
-int int4linear_gemm_fp6_converted(const void *a_conv_d, const void *b_conv_d, void *c_d, int m, int n,
-                                  int k, void *stream)
+}  // extern "C"
+
+namespace {
+
+int fp6_converted_impl(const void *a_conv_d, const void *b_conv_d, void *c_d, int m, int n, int k,
+                       const Epilogue &ep, void *stream)
 {
     if (m < 0 || n < 0 || k < 0 || (k % 8) != 0)
         return INT4LINEAR_ERR_SHAPE;
@@ -504,11 +564,37 @@ int int4linear_gemm_fp6_converted(const void *a_conv_d, const void *b_conv_d, vo
     if (!aligned16(c_d) || ((uintptr_t)a_conv_d & 255) != 0 || ((uintptr_t)b_conv_d & 255) != 0)
         return INT4LINEAR_ERR_ALIGN;
     PerDevice *pd = nullptr;
-    int st = ensure_init(&pd);
+    int st = ensure_init(&pd, true, (hipStream_t)stream);
     if (st != INT4LINEAR_OK)
         return st;
-    hipError_t e = launch_fp6_gemm(a_conv_d, b_conv_d, c_d, m, n, k, Epilogue{}, pd->info, (hipStream_t)stream);
+    hipError_t e = launch_fp6_gemm(a_conv_d, b_conv_d, c_d, m, n, k, ep, pd->info, (hipStream_t)stream);
     return e == hipSuccess ? INT4LINEAR_OK : fail_hip(e);
+}
+
+}  // namespace
+
+extern "C" {
+
+int int4linear_gemm_fp6_converted(const void *a_conv_d, const void *b_conv_d, void *c_d, int m, int n,
+                                  int k, void *stream)
+{
+    return fp6_converted_impl(a_conv_d, b_conv_d, c_d, m, n, k, Epilogue{}, stream);
+}
+
+int int4linear_linear_fp6_converted(const void *x_conv_d, const void *w_conv_d, const int *bias_d,
+                                    const float *row_scale_d, const float *col_scale_d, void *y_d, int out_type,
+                                    int m, int n, int k, void *stream)
+{
+    if (out_type < INT4LINEAR_OUT_S32 || out_type > INT4LINEAR_OUT_BF16)
+        return INT4LINEAR_ERR_UNSUPPORTED;
+    if (out_type == INT4LINEAR_OUT_S32 && (row_scale_d || col_scale_d))
+        return INT4LINEAR_ERR_UNSUPPORTED;  // an int32 output takes a bias only
+    Epilogue ep;
+    ep.bias = bias_d;
+    ep.row_scale = row_scale_d;
+    ep.col_scale = col_scale_d;
+    ep.out = out_type;  // the INT4LINEAR_OUT_* values are the kernels' OutKind values
+    return fp6_converted_impl(x_conv_d, w_conv_d, y_d, m, n, k, ep, stream);
 }
 
 const char *int4linear_kernel_for_shape(int m, int n, int k)
@@ -544,8 +630,10 @@ const char *int4linear_status_string(int status)
         return "requested kernel does not support this shape";
     case INT4LINEAR_ERR_NO_DEVICE:
         return "no usable HIP device";
+    case INT4LINEAR_ERR_NOT_INITIALISED:
+        return "first call on this device came while its stream was being captured: call int4linear_init() before the capture";
     case INT4LINEAR_ERR_SCRATCH:
-        return "shape needs more scratch memory than the static array of int4linear_gemm_s4s4s32_static holds";
+        return "only a kernel with more scratch memory than the static array of int4linear_gemm_s4s4s32_static holds is fast for this shape";
     default:
         return "unknown status";
     }
@@ -561,11 +649,12 @@ size_t int4linear_workspace_bytes(int m, int n, int k)
     const int kernel = pick_kernel(m, n, k, info, g_workspace_limit.load());
     if (kernel == INT4LINEAR_KERNEL_FP6)
         return fp6_workspace_bytes(m, n, k, info);
-    if (kernel == INT4LINEAR_KERNEL_MFMA) {
-        // the split-K form needs the device's CU count: unknown only without a device
+    if (kernel == INT4LINEAR_KERNEL_MFMA || kernel == INT4LINEAR_KERNEL_SKINNY) {
+        // the split-K forms need the device's CU count: unknown only without a device
         if (info.cu_count == 0)
             return 0;
-        const size_t need = mfma_workspace_bytes(m, n, k, info);
+        const size_t need = kernel == INT4LINEAR_KERNEL_MFMA ? mfma_workspace_bytes(m, n, k, info)
+                                                             : skinny_workspace_bytes(m, n, k, info);
         return need <= g_workspace_limit.load() ? need : 0;
     }
     return 0;

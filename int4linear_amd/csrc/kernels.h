@@ -183,6 +183,20 @@ hipError_t skinny_init(const DeviceInfo &dev);
 hipError_t launch_skinny(const void *a, const void *b, void *c, int m, int n, int k,
                          const Epilogue &ep, const DeviceInfo &dev, hipStream_t stream);
 
+// The same kernel split over K across workgroups, for shapes in which a workgroup that owns
+// whole rows of W would pull far more of X than of W (more than 16 rows of X, long K, few
+// rows of W per CU): a workgroup takes a rectangle (rows of W) x (slice of K), stores its
+// partial sums into `workspace` (skinny_workspace_bytes() bytes, 8-byte aligned; 0 = the
+// shape is not split) and counts itself in at `arrivals` (kSkinnyArrivalWords words that are
+// zero before the launch and zero again after it); the last workgroup of a row block to
+// arrive adds the partial sums up, applies the epilogue and stores.  Nobody waits for
+// anybody, and integer sums do not depend on the order of arrival.  Launches that share
+// `workspace` or `arrivals` must not overlap.
+constexpr int kSkinnyArrivalWords = 4096;
+size_t skinny_workspace_bytes(int m, int n, int k, const DeviceInfo &dev);
+hipError_t launch_skinny_ksplit(const void *a, const void *b, void *c, int m, int n, int k, void *workspace,
+                                unsigned *arrivals, const Epilogue &ep, const DeviceInfo &dev, hipStream_t stream);
+
 // Device packer / unpacker, utils/packer.cpp layouts.
 hipError_t launch_pack(const int *src, int *dst, int m, int n, hipStream_t stream);
 hipError_t launch_unpack(const int *src, int *dst, int m, int n, hipStream_t stream);

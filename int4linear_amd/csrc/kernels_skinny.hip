@@ -183,18 +183,31 @@ constexpr int head_bytes(int r, int fmx) { return r * fmx * 1024; }
 // group's sums as soon as it has landed, while the later groups are still in flight, so
 // only the last group's share, the meeting and the stores are exposed after the last byte
 // arrives.
-template <int T, int R, int FMX, bool XDMA, bool RAGGED>
-__global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(const uint8_t *X, const uint8_t *W, int32_t *Y,
-                                                                              v4i dims, Epilogue ep_all)
+//
+// KSPLIT: the grid is (row blocks) x (2 or 4 slices of K, four as launched today); workgroup b takes row block
+// b / slices and slice b % slices of K (an even split into whole tiles; workgroup ids go round
+// the XCDs, so an XCD's workgroups share one or two slices of X), leaves its partial sums
+// in `partial` and counts itself in at `arrivals`; the last of a row block's workgroups to
+// arrive adds them up and stores (see the end of the function).
+template <int T, int R, int FMX, bool XDMA, bool RAGGED, bool KSPLIT>
+__device__ __forceinline__ void skinny_body(const uint8_t *X, const uint8_t *W, int32_t *Y, v4i dims, const Epilogue &ep_all,
+                                            int *partial, unsigned *arrivals)
 {
-    // dims: { M | passes << 8 | S << 16 | plain << 24, N, K, rows_blk } -- one argument instead
-    // of seven: the host's cost of a launch grows with the number of arguments (0.1 us each),
-    // and these launches are short enough for that to show.  `plain` says that ep_all is all
-    // zero, which the storing wave then knows without loading it.
+    static_assert(!(KSPLIT && RAGGED), "slices of K are whole numbers of tiles");
+    // dims: { M | passes << 8 | S << 16 | plain << 24 | log2(slices of K) << 25, N, K, rows_blk } --
+    // one argument instead of seven: the host's cost of a launch grows with the number of
+    // arguments (0.1 us each), and these launches are short enough for that to show.  `plain`
+    // says that ep_all is all zero, which the storing wave then knows without loading it.
     int M = dims[0] & 0xFF, passes = (dims[0] >> 8) & 0xFF;
     const int waves = (dims[0] >> 16) & 0xFF;
     const bool plain = (dims[0] >> 24) & 1;
     const int N = dims[1], K = dims[2], rows_blk = dims[3];
+    const int kslices_log2 = KSPLIT ? (dims[0] >> 25) & 3 : 0;
+    const int kslices = 1 << kslices_log2;
+    const int kslice = KSPLIT ? (int)blockIdx.x & (kslices - 1) : 0;
+    const int row_block = (int)blockIdx.x >> kslices_log2;
+    // first tile of this workgroup's slice of K
+    const int slice_tile0 = KSPLIT ? kslice * (K / kTileK / kslices) : 0;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int kWaveTiles = T * (R + (XDMA ? FMX : 0));
     constexpr int kHead = head_bytes(R, FMX);
@@ -215,7 +228,7 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
     int lane = threadIdx.x & 63;
     int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     unsigned rowbytes = (unsigned)K >> 1;
-    int n0 = blockIdx.x * rows_blk;
+    int n0 = row_block * rows_blk;
     int rows_here = min(rows_blk, N - n0);  // >= 1
     const unsigned lds_base = (unsigned)(size_t)I4L_LDS(lds);
     {
@@ -225,7 +238,7 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
         const unsigned g0 = 16u * (wave & (R - 1));  // the wave's first row group (see `rot`)
         const unsigned lim = (unsigned)(rows_here - 1);
         const int skip0 = RAGGED ? max(0, (wave + 1) * T - K / kTileK) : 0;
-        const uint8_t *base = W + (size_t)n0 * rowbytes + (size_t)(wave * T - skip0) * kTileRowBytes;
+        const uint8_t *base = W + (size_t)n0 * rowbytes + (size_t)(slice_tile0 + wave * T - skip0) * kTileRowBytes;
         const unsigned first_lds = lds_base + kHead + wave * kWaveTiles * kTileBytes;
         dma16_at<true, 0, 0>(base, (unsigned)__umul24(min(g0 + lrow, lim), rowbytes) + ((c8 ^ (lrow >> 1)) << 4), first_lds);
         dma16_at<true, 0, 1024>(base, (unsigned)__umul24(min(g0 + lrow + 8, lim), rowbytes) + ((c8 ^ (4 + (lrow >> 1))) << 4),
@@ -278,7 +291,7 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
     // K's tiles do not fill the last slices, a slice that would run past the end is
     // moved back to end with the last tile, and its first `skip` tiles (someone else's,
     // or all T of them) are loaded like the others but not multiplied.
-    const int first_tile = (pass * waves + wave) * T;
+    const int first_tile = slice_tile0 + (pass * waves + wave) * T;
     if (RAGGED)
         skip = max(0, first_tile + T - K / kTileK);
     const size_t kbyte0 = (size_t)(first_tile - skip) * kTileRowBytes;
@@ -383,7 +396,7 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
         asm volatile("" : "+v"(lane_here));
         const unsigned lrow = (unsigned)lane_here >> 3;
         const unsigned c8 = (unsigned)lane_here & 7;
-        const int first_tile = (pass * waves + wave) * T;
+        const int first_tile = slice_tile0 + (pass * waves + wave) * T;
         const uint8_t *wbase = uniform(W + (size_t)n0 * rowbytes + (size_t)(first_tile - skip) * kTileRowBytes);
         const unsigned g = 16 * ((i + rot) & (R - 1));
         const unsigned off0 = (unsigned)__umul24(min(g + lrow, (unsigned)(rows_here - 1)), rowbytes) + ((c8 ^ (lrow >> 1)) << 4);
@@ -515,27 +528,110 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     const int om = lane >> 2, oj = lane & 3;  // this lane stores Y[om][4 * oj ..+4) of a block
+    // A wave's blocks are j = wave, wave + waves, ...; `sum_of(i, j)` is the i-th of them,
+    // complete.  Unsplit: read from LDS.  Split over K: read back from all slices' slabs.
+    constexpr int kBlocks = R * FMX;
+    constexpr int kMine = KSPLIT ? (kBlocks + 3) / 4 : 1;  // blocks per wave when split (at least four waves: the host checks)
+    v4i gathered[kMine];
+    if constexpr (KSPLIT) {
+        // The exchange.  Slab (row block, slice) of `partial` holds the workgroup's kBlocks
+        // blocks of 256 sums, a lane's four as two 64-bit words at 64 * h + lane of the block.
+        // The stores and the loads are relaxed atomic operations at device scope, which on
+        // this device are plain accesses that go through to (come from) the level all
+        // workgroups share; the stores have been acknowledged before the wave counts itself
+        // in, so whoever sees the last increment of a counter finds every slice's slab.  The
+        // counter is that of (row block, wave): the waves with one number hold the same blocks
+        // in every slice's workgroup, so the last of them to arrive adds those blocks up and
+        // stores them, and puts the counter back to zero for the next launch.  Nobody waits
+        // for anybody; integer sums do not depend on who arrives when.  All of a wave's
+        // operations of a kind go out together: a trip to memory costs far more than they do.
+        typedef unsigned long long u64;
+        u64 *const slabs = (u64 *)partial + (size_t)row_block * kslices * kBlocks * 128 + lane;
+        u64 *const mine_at = slabs + (size_t)kslice * kBlocks * 128;
+#pragma unroll
+        for (int i = 0; i < kMine; ++i) {
+            const int j = wave + i * waves;
+            if (j < kBlocks) {
+                const int *mine_of = sums + j * 256 + 16 * oj + om;
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+                    __hip_atomic_store(mine_at + j * 128 + 64 * h,
+                                       (u64)(unsigned)mine_of[128 * h] | ((u64)(unsigned)mine_of[128 * h + 64] << 32), __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        unsigned *const counter = arrivals + row_block * waves + wave;
+        unsigned before = 0;
+        if (lane == 0)
+            before = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        before = uniform(before);
+        if (before != (unsigned)(kslices - 1))
+            return;
+        if (lane == 0)
+            __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        u64 got[kMine][4][2];
+#pragma unroll
+        for (int i = 0; i < kMine; ++i)
+#pragma unroll
+            for (int p = 0; p < 4; ++p)
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const int j = wave + i * waves;
+                    got[i][p][h] = (j < kBlocks && p < kslices)
+                                       ? __hip_atomic_load(slabs + ((size_t)p * kBlocks + j) * 128 + 64 * h, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                                       : 0ull;
+                }
+#pragma unroll
+        for (int i = 0; i < kMine; ++i) {
+            gathered[i] = (v4i){0, 0, 0, 0};
+#pragma unroll
+            for (int p = 0; p < 4; ++p)
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    gathered[i][2 * h] += (int)(unsigned)got[i][p][h];
+                    gathered[i][2 * h + 1] += (int)(unsigned)(got[i][p][h] >> 32);
+                }
+        }
+    }
+    auto sum_of = [&](int i, int j) -> v4i {
+        if constexpr (KSPLIT) {
+            return gathered[i];
+        } else {
+            const int *mine_of = sums + j * 256 + 16 * oj + om;
+            return (v4i){mine_of[0], mine_of[64], mine_of[128], mine_of[192]};
+        }
+    };
+    // f(i, j) for each of the wave's blocks; unrolled when split (the sums are in registers).
+    auto for_my_blocks = [&](auto &&f) {
+        if constexpr (KSPLIT) {
+#pragma unroll
+            for (int i = 0; i < kMine; ++i)
+                if (wave + i * waves < kBlocks)
+                    f(i, wave + i * waves);
+        } else {
+#pragma unroll 1
+            for (int j = wave; j < kBlocks; j += waves)
+                f(0, j);
+        }
+    };
     if (plain && ((N | rows_here) & 3) == 0) {
         // Nothing to load or to convert, and a lane's four outputs exist together or not at
         // all: the path that ends the kernel in the common case, kept to a few instructions.
-#pragma unroll 1
-        for (int j = wave; j < R * FMX; j += waves) {  // block j: row group j / FMX of W, j % FMX of X
+        for_my_blocks([&](int i, int j) {  // block j: row group j / FMX of W, j % FMX of X
             const int rg = j / FMX, f = j % FMX;
-            const int *mine_of = sums + j * 256 + 16 * oj + om;
-            const v4i sum = {mine_of[0], mine_of[64], mine_of[128], mine_of[192]};
+            const v4i sum = sum_of(i, j);
             if (f * 16 + om < M && rg * 16 + 4 * oj < rows_here)
                 *(v4i *)(Y + (size_t)(f * 16 + om) * N + n0 + rg * 16 + 4 * oj) = sum;
-        }
+        });
         return;
     }
     // (the epilogue's operands are first looked at here, not ahead of the loads)
     Epilogue ep = ep_all;
     asm volatile("" : "+s"(ep.bias), "+s"(ep.row_scale), "+s"(ep.col_scale), "+s"(ep.out));
-#pragma unroll 1
-    for (int j = wave; j < R * FMX; j += waves) {
+    for_my_blocks([&](int i, int j) {
         const int rg = j / FMX, f = j % FMX;
-        const int *mine_of = sums + j * 256 + 16 * oj + om;
-        v4i sum = {mine_of[0], mine_of[64], mine_of[128], mine_of[192]};
+        v4i sum = sum_of(i, j);
         const int m = f * 16 + om;
         const int nb = rg * 16 + 4 * oj;  // within the workgroup's rows
         if (m < M) {
@@ -549,7 +645,22 @@ __global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(co
                 store_out4<half()>(Y, (size_t)m * N + n0 + nb, sum, rows_here - nb, nb + 3 < rows_here && ((N | n0) & 3) == 0);
             });
         }
-    }
+    });
+}
+
+template <int T, int R, int FMX, bool XDMA, bool RAGGED>
+__global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_kernel(const uint8_t *X, const uint8_t *W, int32_t *Y,
+                                                                              v4i dims, Epilogue ep_all)
+{
+    skinny_body<T, R, FMX, XDMA, RAGGED, false>(X, W, Y, dims, ep_all, nullptr, nullptr);
+}
+
+template <int T, int R, int FMX, bool XDMA>
+__global__ __launch_bounds__(max_threads(T, R, FMX, XDMA)) void skinny_ksplit_kernel(const uint8_t *X, const uint8_t *W, int32_t *Y,
+                                                                                     v4i dims, Epilogue ep_all, int *partial,
+                                                                                     unsigned *arrivals)
+{
+    skinny_body<T, R, FMX, XDMA, false, true>(X, W, Y, dims, ep_all, partial, arrivals);
 }
 
 // ---- long-W form: many 16-row groups of W per CU, FMX 16-row groups of X.
@@ -959,13 +1070,45 @@ bool make_plan(int m, int n, int k, int cu_count, Plan &p)
     return make_plan(m, n, k, cu_count, false, p) || make_plan(m, n, k, cu_count, true, p);
 }
 
+// The split over K across workgroups exists for more than 32 rows of X and several row groups
+// of W per workgroup (the shapes it is for; every instantiation costs build time).
+constexpr bool ksplit_variant_exists(int t, int r, int fmx, bool xdma)
+{
+    return variant_exists(t, r, fmx, xdma) && fmx >= 3 && r >= 2;
+}
+
+// Where a launch that is split over K keeps its partial sums and counts its arrivals.
+struct KSplit {
+    int slices = 1;
+    int *partial = nullptr;
+    unsigned *arrivals = nullptr;
+};
+
 template <int T, int R, int FMX, bool XDMA>
 hipError_t launch_plan(const Plan &p, const void *a, const void *b, void *c, int m, int n, int k,
-                       const Epilogue &ep, hipStream_t stream)
+                       const Epilogue &ep, hipStream_t stream, const KSplit &split = KSplit{})
 {
     if constexpr (!variant_exists(T, R, FMX, XDMA)) {
         return p.s == 0 ? hipSuccess : hipErrorInvalidConfiguration;  // never planned
     } else {
+    if constexpr (ksplit_variant_exists(T, R, FMX, XDMA)) {
+        auto kern = skinny_ksplit_kernel<T, R, FMX, XDMA>;
+        if (p.s == 0) {  // set-up call, for both forms
+            const hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
+            if (e != hipSuccess)
+                return e;
+        } else if (split.slices > 1) {
+            const unsigned row_blocks = (unsigned)((n + p.rows_blk - 1) / p.rows_blk);
+            const int plain = !ep.bias && !ep.row_scale && !ep.col_scale && !ep.out;
+            kern<<<row_blocks * split.slices, p.s * 64, p.lds, stream>>>(
+                (const uint8_t *)a, (const uint8_t *)b, (int32_t *)c,
+                (v4i){m | (p.passes << 8) | (p.s << 16) | (plain << 24) | ((split.slices == 4 ? 2 : 1) << 25), n, k, p.rows_blk}, ep, split.partial,
+                split.arrivals);
+            return hipGetLastError();
+        }
+    } else if (split.slices > 1) {
+        return hipErrorInvalidConfiguration;
+    }
     auto kern = p.ragged ? skinny_kernel<T, R, FMX, XDMA, true> : skinny_kernel<T, R, FMX, XDMA, false>;
     if (p.s == 0)  // set-up call: raise the dynamic-LDS limit of this instantiation
         return hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
@@ -991,11 +1134,11 @@ hipError_t launch_plan(const Plan &p, const void *a, const void *b, void *c, int
 
 template <int T, bool XDMA>
 hipError_t dispatch_rf(const Plan &p, const void *a, const void *b, void *c, int m, int n, int k,
-                       const Epilogue &ep, hipStream_t stream)
+                       const Epilogue &ep, hipStream_t stream, const KSplit &split)
 {
 #define I4L_CASE(R_, F_)                                                      \
     if (p.r == R_ && p.fmx == F_)                                             \
-        return launch_plan<T, R_, F_, XDMA>(p, a, b, c, m, n, k, ep, stream);
+        return launch_plan<T, R_, F_, XDMA>(p, a, b, c, m, n, k, ep, stream, split);
     I4L_CASE(4, 1) I4L_CASE(2, 1) I4L_CASE(1, 1)
     I4L_CASE(4, 2) I4L_CASE(2, 2) I4L_CASE(1, 2)
     I4L_CASE(4, 3) I4L_CASE(2, 3) I4L_CASE(1, 3)
@@ -1010,17 +1153,17 @@ namespace {
 
 template <bool XDMA>
 hipError_t dispatch_t(const Plan &p, const void *a, const void *b, void *c, int m, int n, int k,
-                      const Epilogue &ep, hipStream_t stream)
+                      const Epilogue &ep, hipStream_t stream, const KSplit &split = KSplit{})
 {
     switch (p.t) {
     case 1:
-        return dispatch_rf<1, XDMA>(p, a, b, c, m, n, k, ep, stream);
+        return dispatch_rf<1, XDMA>(p, a, b, c, m, n, k, ep, stream, split);
     case 2:
-        return dispatch_rf<2, XDMA>(p, a, b, c, m, n, k, ep, stream);
+        return dispatch_rf<2, XDMA>(p, a, b, c, m, n, k, ep, stream, split);
     case 3:
-        return dispatch_rf<3, XDMA>(p, a, b, c, m, n, k, ep, stream);
+        return dispatch_rf<3, XDMA>(p, a, b, c, m, n, k, ep, stream, split);
     case 4:
-        return dispatch_rf<4, XDMA>(p, a, b, c, m, n, k, ep, stream);
+        return dispatch_rf<4, XDMA>(p, a, b, c, m, n, k, ep, stream, split);
     default:
         return hipErrorInvalidConfiguration;
     }
@@ -1176,7 +1319,49 @@ bool skinny_preferred(int m, int n, int k, const DeviceInfo &)
 
 namespace {
 
-// The plan of the shape a host thread asked for last: a decode loop calls with a handful of
+// The split over K across workgroups.  Whole rows of W per workgroup mean that every
+// workgroup pulls all of X: with N = 4096 on 256 CUs that is 16 rows of W against all M rows
+// of X, four times the workgroup's share of W at M = 64, and every workgroup widens all of
+// it.  A workgroup that takes four times the rows and a quarter of K pulls (and widens) a
+// quarter of X for the same bytes of W.  What it costs is the exchange at the end -- partial
+// sums to memory, an arrival counter, the last workgroup to arrive reading them back: three
+// trips to memory that nothing overlaps, about 3 us while the other workgroups still stream
+// (measured: 64 x 4096 x 14336 takes 10.3 us split four ways with the exchange left out and
+// 13.3 us with it, against 14.1 us unsplit; one returning atomic addition per output
+// element instead of the slabs is a single trip but is bound by the rate of the atomic
+// units, 3.5 us for the same shape; up to 32 rows of X the gain is smaller than that, and
+// with up to 16 rows there is none even with the exchange left out).  So: 33 to 64 rows
+// of X, K in whole tiles that split evenly into four slices of at least 14 tiles
+// (K >= 14336; at 8192 the exchange costs more than the split saves), at most 64 rows per
+// workgroup.
+bool make_ksplit_plan(int m, int n, int k, int cu_count, Plan &p, int &slices)
+{
+    constexpr int kSlices = 4, kMinTilesPerSlice = 14;
+    if (m <= 32 || m > 64 || k % kTileK != 0 || cu_count <= 0)
+        return false;
+    const int tiles = k / kTileK;
+    const int fmx = (m + 15) / 16;
+    const long row_blocks_max = cu_count / kSlices;
+    if (tiles % kSlices != 0 || tiles / kSlices < kMinTilesPerSlice || row_blocks_max < 1)
+        return false;
+    const long per_block = (n + row_blocks_max - 1) / row_blocks_max;
+    const int rows_blk = (int)((per_block + 7) / 8 * 8);
+    if (rows_blk > 64)
+        return false;  // more rows than one round of workgroups holds: the unsplit form's case
+    int r = 1;
+    while (16 * r < rows_blk)
+        r <<= 1;
+    if (r < 2 || !fit(tiles / kSlices, fmx, r, false, p) || !ksplit_variant_exists(p.t, p.r, p.fmx, p.xdma))
+        return false;
+    const long row_blocks = (n + rows_blk - 1) / rows_blk;
+    if (p.s < 4 || row_blocks * p.s > kSkinnyArrivalWords)
+        return false;
+    p.rows_blk = rows_blk;
+    slices = kSlices;
+    return true;
+}
+
+// The plans of the shape a host thread asked for last: a decode loop calls with a handful of
 // shapes over and over, and next to a kernel of a few microseconds the plan search (some
 // hundred candidate splits) is not free.
 struct PlanCache {
@@ -1184,22 +1369,57 @@ struct PlanCache {
     int kind = 0;  // 1: long-W form, 2: tiled form, 3: neither
     StreamPlan sp;
     Plan p;
+    int slices = 1;  // > 1: the split over K across workgroups applies, with plan `split`
+    Plan split;
+    size_t split_bytes = 0;
 };
 thread_local PlanCache t_plan;
 
-}  // namespace
-
-hipError_t launch_skinny(const void *a, const void *b, void *c, int m, int n, int k,
-                         const Epilogue &ep, const DeviceInfo &dev, hipStream_t stream)
+PlanCache &plans_for(int m, int n, int k, const DeviceInfo &dev)
 {
     PlanCache &pc = t_plan;
     if (pc.m != m || pc.n != n || pc.k != k || pc.cus != dev.cu_count) {
         pc.kind = make_stream_plan(m, n, k, dev.cu_count, pc.sp) ? 1 : make_plan(m, n, k, dev.cu_count, pc.p) ? 2 : 3;
+        pc.slices = 1;
+        pc.split_bytes = 0;
+        if (pc.kind == 2 && make_ksplit_plan(m, n, k, dev.cu_count, pc.split, pc.slices)) {
+            const size_t row_blocks = (size_t)((n + pc.split.rows_blk - 1) / pc.split.rows_blk);
+            pc.split_bytes = row_blocks * pc.slices * pc.split.r * pc.split.fmx * 1024;
+        } else {
+            pc.slices = 1;
+        }
         pc.m = m;
         pc.n = n;
         pc.k = k;
         pc.cus = dev.cu_count;
     }
+    return pc;
+}
+
+}  // namespace
+
+size_t skinny_workspace_bytes(int m, int n, int k, const DeviceInfo &dev)
+{
+    if (m <= 32 || !skinny_supports(m, n, k))  // (the common decode call: not even a look at the cache)
+        return 0;
+    return plans_for(m, n, k, dev).split_bytes;
+}
+
+hipError_t launch_skinny_ksplit(const void *a, const void *b, void *c, int m, int n, int k, void *workspace,
+                                unsigned *arrivals, const Epilogue &ep, const DeviceInfo &dev, hipStream_t stream)
+{
+    PlanCache &pc = plans_for(m, n, k, dev);
+    if (pc.slices <= 1 || !workspace || !arrivals)
+        return launch_skinny(a, b, c, m, n, k, ep, dev, stream);
+    const KSplit split{pc.slices, (int *)workspace, arrivals};
+    return pc.split.xdma ? dispatch_t<true>(pc.split, a, b, c, m, n, k, ep, stream, split)
+                         : dispatch_t<false>(pc.split, a, b, c, m, n, k, ep, stream, split);
+}
+
+hipError_t launch_skinny(const void *a, const void *b, void *c, int m, int n, int k,
+                         const Epilogue &ep, const DeviceInfo &dev, hipStream_t stream)
+{
+    PlanCache &pc = plans_for(m, n, k, dev);
     if (pc.kind == 1)
         return dispatch_stream(pc.sp, a, b, c, m, n, k, ep, stream);
     if (pc.kind == 2)

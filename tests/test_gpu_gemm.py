@@ -110,6 +110,9 @@ def test_cfg4_decode(gpu, host_threads, m, n, k):
     (64, 4096, 14336), (32, 4100, 14336), (16, 14336, 14336), (64, 500, 20480), (8, 700, 32768), (48, 1000, 12288),
     # ... with several row groups of W and of X (later groups issued one ahead, in every pass)
     (32, 8200, 32768), (64, 8200, 20480), (48, 14336, 12288),
+    # 33 to 64 rows of X, few rows of W per CU, long K: split four ways over K across workgroups under
+    # automatic dispatch (whole row blocks, a ragged last one, fewer row blocks than a quarter of the CUs)
+    (48, 4096, 14336), (33, 4000, 14336), (64, 3000, 14336), (64, 2048, 28672), (40, 2000, 16384), (50, 2100, 57344),
     # more than 64 rows of X: runs of 64, one launch each (only when the kernel is asked for by name)
     (65, 4096, 4096), (128, 14336, 4096), (100, 3000, 2048), (96, 14336, 512), (128, 600, 14336),
     (200, 520, 1024), (130, 20000, 4096),
@@ -134,6 +137,129 @@ def test_skinny_plans(gpu, host_threads, m, n, k):
         got = helpers.run_gemm(xp, wp, m, n, k, kernel=kern)
         bad = np.argwhere(got != want)
         assert bad.size == 0, f"kernel={kern}: {len(bad)} mismatches, first at {tuple(bad[0])}"
+
+
+def test_decode_split_over_k_across_workgroups(gpu, host_threads):
+    """The shapes of the weight-streaming kernel whose workgroups take a slice of K each and
+    exchange partial sums through the workspace: two shapes in turn, new data every call (the
+    arrival counters must be back at zero after every launch), on alternating streams without
+    host synchronisation (the library orders users of the workspace), and under graph capture
+    (no workspace there: the unsplit form, same result)."""
+    import torch
+
+    import int4linear_amd as lib
+
+    shapes = [(64, 4096, 14336), (40, 2000, 16384)]
+    for (m, n, k) in shapes:
+        assert lib.kernel_for_shape(m, n, k) == "skinny" and lib.workspace_bytes(m, n, k) > 0, (m, n, k)
+    assert lib.workspace_bytes(16, 4096, 14336) == 0 and lib.workspace_bytes(64, 4096, 8192) == 0
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    cases = []
+    for i in range(6):
+        m, n, k = shapes[i % 2]
+        x = helpers.normal_s4(2100 + i, m, k)
+        w = helpers.uniform_s4(2200 + i, n, k)
+        cases.append((m, n, k, helpers.to_device_bytes(helpers.pack_bytes(x)), helpers.to_device_bytes(helpers.pack_bytes(w)),
+                      torch.full((m, n), -1, dtype=torch.int32, device="cuda:0"), oracle.linear_ref(x, w, threads=host_threads)))
+    torch.cuda.synchronize()
+    for rep in range(3):
+        for i, (m, n, k, xd, wd, yd, _) in enumerate(cases):
+            lib.gemm_s4s4s32(xd, wd, yd, m, n, k, stream=streams[(i + rep) % 2].cuda_stream)
+    torch.cuda.synchronize()
+    for i, (m, n, k, _, _, yd, want) in enumerate(cases):
+        assert np.array_equal(yd.cpu().numpy(), want), f"case {i} {(m, n, k)}"
+    # captured: automatic dispatch must not touch the workspace
+    m, n, k, xd, wd, yd, want = cases[0]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        lib.gemm_s4s4s32(xd, wd, yd, m, n, k)
+    for rep in range(2):
+        yd.fill_(-1)
+        lib.release_workspace()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(yd.cpu().numpy(), want), f"captured, replay {rep}"
+
+
+@pytest.mark.parametrize("m, n, k", [(1024, 2048, 4096), (777, 33, 1152), (300, 520, 512)])
+def test_epilogue_on_fp6_converted_operands(gpu, host_threads, m, n, k):
+    """int4linear_linear_fp6_converted: the bias add and the scaled float / half / bfloat16
+    outputs on caller-owned converted operands, bit for bit against the oracle's epilogue."""
+    import torch
+
+    import int4linear_amd as lib
+
+    rng = np.random.default_rng(m * 7 + n)
+    x = helpers.normal_s4(2300 + m, m, k)
+    w = helpers.uniform_s4(2400 + n, n, k)
+    prod = oracle.linear_ref(x, w, threads=host_threads)
+    bias = rng.integers(-100000, 100000, size=n, dtype=np.int32)
+    rs = (rng.uniform(0.01, 2.0, size=m) * 2.0 ** -9).astype(np.float32)
+    cs = rng.uniform(0.01, 2.0, size=n).astype(np.float32)
+    xd = helpers.to_device_bytes(helpers.pack_bytes(x))
+    wd = helpers.to_device_bytes(helpers.pack_bytes(w))
+    xc = torch.empty(lib.fp6_operand_bytes(m, k), dtype=torch.uint8, device="cuda:0")
+    wc = torch.empty(lib.fp6_operand_bytes(n, k), dtype=torch.uint8, device="cuda:0")
+    lib.fp6_convert(xd, xc, m, k)
+    lib.fp6_convert(wd, wc, n, k)
+    bd, rd, cd = (torch.from_numpy(a).to("cuda:0") for a in (bias, rs, cs))
+    y = torch.full((m, n), 0x7BADBAD, dtype=torch.int32, device="cuda:0")
+    lib.linear_fp6_converted(xc, wc, bd, None, None, y, "s32", m, n, k)
+    assert np.array_equal(y.cpu().numpy(), oracle.epilogue(prod, bias)), "s32"
+    lib.linear_fp6_converted(xc, wc, None, None, None, y, "s32", m, n, k)
+    assert np.array_equal(y.cpu().numpy(), prod), "s32 without bias"
+    yf = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda:0")
+    lib.linear_fp6_converted(xc, wc, bd, rd, cd, yf, "f32", m, n, k)
+    assert np.array_equal(yf.cpu().numpy().view(np.int32), oracle.epilogue(prod, bias, rs, cs, f32=True).view(np.int32)), "f32"
+    lib.linear_fp6_converted(xc, wc, None, rd, None, yf, "f32", m, n, k)
+    assert np.array_equal(yf.cpu().numpy().view(np.int32), oracle.epilogue(prod, None, rs, None, f32=True).view(np.int32)), "f32 row scale"
+    for kind in ("f16", "bf16"):
+        y16 = torch.full((m * n + 256,), 0x7BAD, dtype=torch.int16, device="cuda:0")
+        lib.linear_fp6_converted(xc, wc, bd, rd, cd, y16, kind, m, n, k)
+        got = y16.cpu().numpy().view(np.uint16)
+        assert np.array_equal(got[:m * n].reshape(m, n), oracle.epilogue(prod, bias, rs, cs, out=kind)), kind
+        assert np.all(got[m * n:] == 0x7BAD), f"{kind}: wrote past the output"
+    # an int32 output takes no scales; an unknown output type is refused
+    with pytest.raises(lib.Int4LinearError) as refused:
+        lib.linear_fp6_converted(xc, wc, bd, rd, None, y, "s32", m, n, k)
+    assert refused.value.status == 5
+    from int4linear_amd import _lib
+    assert _lib.load().int4linear_linear_fp6_converted(xc.data_ptr(), wc.data_ptr(), None, None, None, y.data_ptr(), 4, m, n, k, None) == 5
+
+
+def test_first_call_inside_a_capture_is_refused(gpu):
+    """Set-up must not happen inside a graph capture: a process whose first library call comes
+    while its stream is capturing gets INT4LINEAR_ERR_NOT_INITIALISED (and may call again after
+    int4linear_init()).  Needs a process of its own: this one has set the device up long ago."""
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    code = (
+        "import sys, ctypes, torch\n"
+        "sys.path.insert(0, %r)\n"
+        "from int4linear_amd import _lib\n"
+        "L = _lib.load()\n"
+        "x = torch.zeros(16 * 512, dtype=torch.uint8, device='cuda:0'); w = torch.zeros(1024 * 512, dtype=torch.uint8, device='cuda:0')\n"
+        "y = torch.zeros((16, 1024), dtype=torch.int32, device='cuda:0')\n"
+        "torch.cuda.synchronize()\n"
+        "s = torch.cuda.Stream()\n"
+        "g = torch.cuda.CUDAGraph()\n"
+        "with torch.cuda.graph(g, stream=s):\n"
+        "    st = L.int4linear_gemm_s4s4s32(x.data_ptr(), w.data_ptr(), y.data_ptr(), 16, 1024, 1024, ctypes.c_void_p(s.cuda_stream))\n"
+        "print('captured call:', st, L.int4linear_status_string(st).decode())\n"
+        "assert st == 8, st\n"
+        "assert L.int4linear_init() == 0\n"
+        "g2 = torch.cuda.CUDAGraph()\n"
+        "with torch.cuda.graph(g2, stream=s):\n"
+        "    st = L.int4linear_gemm_s4s4s32(x.data_ptr(), w.data_ptr(), y.data_ptr(), 16, 1024, 1024, ctypes.c_void_p(s.cuda_stream))\n"
+        "assert st == 0, st\n"
+        "y.fill_(-1); g2.replay(); torch.cuda.synchronize()\n"
+        "assert int(y.abs().sum()) == 0\n"
+        "print('ok')\n"
+    ) % str(Path(__file__).resolve().parent.parent)
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and "ok" in r.stdout, r.stdout + r.stderr
 
 
 @pytest.mark.parametrize("m, n, k", [(300, 520, 512), (1, 1, 128), (1024, 2048, 4096), (777, 33, 1152)])
@@ -189,6 +315,8 @@ def test_ragged_k_runs_on_the_fp6_kernel(gpu, host_threads, m, n, k):
     (33, 70, 72, ("auto", "simple", "fp6")),
     (9, 1000, 1920, ("skinny",)),           # the fallback streaming kernel
     (2048, 2304, 1024, ("auto", "mfma")),   # 72 tiles of 256 x 256, several per workgroup
+    (64, 4096, 14336, ("auto",)),           # decode split over K across workgroups: the last arrival applies the epilogue
+    (40, 3000, 14336, ("auto", "skinny")),  # ... with a ragged last row block, against the unsplit form
 ])
 def test_linear_with_epilogue(gpu, host_threads, m, n, k, kernels):
     import torch

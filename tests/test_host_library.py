@@ -45,8 +45,8 @@ def test_reference_cxx_entry_points_exported():
 
 def test_status_strings():
     L = _lib.load()
-    seen = {L.int4linear_status_string(s).decode() for s in range(0, 7)}
-    assert len(seen) == 7 and "ok" in seen
+    seen = {L.int4linear_status_string(s).decode() for s in range(0, 9)}
+    assert len(seen) == 9 and "ok" in seen and "unknown status" not in seen
     assert L.int4linear_status_string(99).decode() == "unknown status"
 
 

@@ -39,6 +39,7 @@ PAIRS = [
     ("fp6 then int8 split-K", (2048, 8192, 8192), "fp6", (128, 4096, 14336), "mfma"),
     ("int8 split-K, 128^2 then 64^2 slices", (512, 4096, 14336), "mfma", (200, 136, 16384), "mfma"),
     ("fp6 with ragged K then a tiny one", (1000, 3000, 4104), "fp6", (40, 56, 4104), "fp6"),
+    ("decode split over K, then a smaller one", (64, 4096, 14336), "skinny", (40, 2000, 16384), "skinny"),
 ]
 
 
@@ -73,15 +74,32 @@ def test_static_kernels_without_scratch(gpu):
         assert torch.equal(got, want), shape
 
 
-def test_static_rejects_oversize(gpu):
-    """A shape whose kernel would need more than the array holds is refused with status 7
-    before anything is enqueued; the output is left alone."""
+def test_static_falls_back_or_rejects_oversize(gpu):
+    """A shape whose fast kernel would need more scratch than the array holds runs on the
+    kernels that need none (as under graph capture); only when that would leave a large
+    problem to the scalar kernel (K not a multiple of 128) is it refused, with status 7, before
+    anything is enqueued and with the output left alone."""
     import torch
 
     import int4linear_amd as lib
     from int4linear_amd import _lib
 
-    m, n, k = 16384, 16384, 8192  # FP6 operands alone: 192 MiB
+    m, n, k = 12288, 12288, 8192  # FP6 operands: 144 MiB
+    assert lib.kernel_for_shape(m, n, k) == "fp6"
+    assert lib.workspace_bytes(m, n, k) > lib.api.STATIC_SCRATCH_BYTES
+    g = torch.Generator(device="cuda:0")
+    g.manual_seed(77)
+    xd = torch.randint(0, 256, (m * k // 2,), dtype=torch.uint8, device="cuda:0", generator=g)
+    wd = torch.randint(0, 256, (n * k // 2,), dtype=torch.uint8, device="cuda:0", generator=g)
+    want = torch.full((m, n), POISON, dtype=torch.int32, device="cuda:0")
+    got = torch.full((m, n), POISON, dtype=torch.int32, device="cuda:0")
+    lib.gemm_s4s4s32(xd, wd, want, m, n, k)
+    lib.gemm_s4s4s32_static(xd, wd, got, m, n, k)   # the int8 kernel: no scratch
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    del want, got
+
+    k = 8200  # K % 128 != 0: only the FP6 kernel is fast, and its operands do not fit
     assert lib.kernel_for_shape(m, n, k) == "fp6"
     assert lib.workspace_bytes(m, n, k) > lib.api.STATIC_SCRATCH_BYTES
     xd = torch.zeros(m * k // 2, dtype=torch.uint8, device="cuda:0")
@@ -106,7 +124,8 @@ def test_static_entry_in_a_graph(gpu):
 
     import int4linear_amd as lib
 
-    shapes = [(2304, 4096, 3072), (128, 4096, 14336)]  # FP6 kernel; int8 split over K
+    shapes = [(2304, 4096, 3072), (128, 4096, 14336), (64, 4096, 14336)]  # FP6 kernel; int8 split over K; decode split over K
+    lib.init()  # set-up does not belong inside a capture (a first call there is refused)
     bufs = []
     for (m, n, k) in shapes:
         bufs.append((torch.zeros(m * k // 2, dtype=torch.uint8, device="cuda:0"),
