@@ -112,10 +112,16 @@ __device__ __forceinline__ void static_for(F &&f)
     }(std::make_integer_sequence<int, N>{});
 }
 
-// LDS slot (16 bytes) of chunk c of tile row r: c ^ ((r >> 1) & 7).  Rows are 128 B apart,
+// LDS slot (16 bytes) of chunk c of tile row r: c ^ ((r >> 1) & MASK).  Rows are 128 B apart,
 // so the sixteen lanes that read one chunk of rows 0..15 hit sixteen different 16-byte
-// bank groups of the 256-byte bank window.
-__device__ __forceinline__ int slot_swizzle(int r) { return (r >> 1) & 7; }
+// bank groups of the 256-byte bank window.  Which mask leaves a 16-byte read per lane free of
+// bank conflicts depends on which chunks the four 16-lane groups of a wave read together
+// (measured with a loop of such reads, cycles per read against 57 for a linear one): four
+// neighbouring chunks of one tile (the plain fragment order) want mask 7 (57; mask 3: 61),
+// chunks j and 4 + j of two tiles (the order that goes with the transposed X loads) want
+// mask 3 (57; mask 7: 61).
+template <int MASK = 7>
+__device__ __forceinline__ int slot_swizzle(int r) { return (r >> 1) & MASK; }
 
 // Waits until at most n of this wave's vector-memory operations are outstanding
 // (they complete in issue order).  n is a compile-time constant at every call site after
@@ -211,6 +217,7 @@ __device__ __forceinline__ void skinny_body(const uint8_t *X, const uint8_t *W, 
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int kWaveTiles = T * (R + (XDMA ? FMX : 0));
     constexpr int kHead = head_bytes(R, FMX);
+    constexpr int kSwMask = (!XDMA && T % 2 == 0) ? 3 : 7;  // the slot swizzle that suits the form's fragment reads
     // Row groups of W whose loads are in flight ahead of the one being multiplied.  With one
     // row group of X a wave issues everything at once.  With more, a wave has X (16 * FMX
     // rows of its K slice) to fetch as well, the CU's queue of outstanding loads fills up, a
@@ -240,8 +247,8 @@ __device__ __forceinline__ void skinny_body(const uint8_t *X, const uint8_t *W, 
         const int skip0 = RAGGED ? max(0, (wave + 1) * T - K / kTileK) : 0;
         const uint8_t *base = W + (size_t)n0 * rowbytes + (size_t)(slice_tile0 + wave * T - skip0) * kTileRowBytes;
         const unsigned first_lds = lds_base + kHead + wave * kWaveTiles * kTileBytes;
-        dma16_at<true, 0, 0>(base, (unsigned)__umul24(min(g0 + lrow, lim), rowbytes) + ((c8 ^ (lrow >> 1)) << 4), first_lds);
-        dma16_at<true, 0, 1024>(base, (unsigned)__umul24(min(g0 + lrow + 8, lim), rowbytes) + ((c8 ^ (4 + (lrow >> 1))) << 4),
+        dma16_at<true, 0, 0>(base, (unsigned)__umul24(min(g0 + lrow, lim), rowbytes) + ((c8 ^ ((lrow >> 1) & kSwMask)) << 4), first_lds);
+        dma16_at<true, 0, 1024>(base, (unsigned)__umul24(min(g0 + lrow + 8, lim), rowbytes) + ((c8 ^ ((4 + (lrow >> 1)) & kSwMask)) << 4),
                                 first_lds);
     }
     asm volatile("" : "+v"(lane), "+s"(wave), "+s"(rowbytes), "+s"(n0), "+s"(rows_here), "+s"(M), "+s"(passes));
@@ -258,7 +265,7 @@ __device__ __forceinline__ void skinny_body(const uint8_t *X, const uint8_t *W, 
     // 4*s + l/16 (32 nibbles: even ones feed one MFMA, odd ones the next).
     const int fr = lane & 15;
     const int fg = lane >> 4;
-    const int sw = slot_swizzle(fr);
+    const int sw = slot_swizzle<kSwMask>(fr);
 
     // With X in registers and an even T the X loads are made in a form the memory pipeline
     // takes at full rate (every quad of lanes reads 64 contiguous bytes of one row; the
@@ -286,7 +293,7 @@ __device__ __forceinline__ void skinny_body(const uint8_t *X, const uint8_t *W, 
     asm volatile("" : "+v"(lane_here));
     const unsigned lrow = (unsigned)lane_here >> 3;
     const unsigned c8 = (unsigned)lane_here & 7;
-    const unsigned chunk[2] = {(c8 ^ (lrow >> 1)) << 4, (c8 ^ (4 + (lrow >> 1))) << 4};
+    const unsigned chunk[2] = {(c8 ^ ((lrow >> 1) & kSwMask)) << 4, (c8 ^ ((4 + (lrow >> 1)) & kSwMask)) << 4};
     // This wave's slice of every row: T tiles from tile (pass * S + wave) * T on.  When
     // K's tiles do not fill the last slices, a slice that would run past the end is
     // moved back to end with the last tile, and its first `skip` tiles (someone else's,
@@ -399,9 +406,9 @@ __device__ __forceinline__ void skinny_body(const uint8_t *X, const uint8_t *W, 
         const int first_tile = slice_tile0 + (pass * waves + wave) * T;
         const uint8_t *wbase = uniform(W + (size_t)n0 * rowbytes + (size_t)(first_tile - skip) * kTileRowBytes);
         const unsigned g = 16 * ((i + rot) & (R - 1));
-        const unsigned off0 = (unsigned)__umul24(min(g + lrow, (unsigned)(rows_here - 1)), rowbytes) + ((c8 ^ (lrow >> 1)) << 4);
+        const unsigned off0 = (unsigned)__umul24(min(g + lrow, (unsigned)(rows_here - 1)), rowbytes) + ((c8 ^ ((lrow >> 1) & kSwMask)) << 4);
         const unsigned off1 = (unsigned)__umul24(min(g + lrow + 8, (unsigned)(rows_here - 1)), rowbytes) +
-                              ((c8 ^ (4 + (lrow >> 1))) << 4);
+                              ((c8 ^ ((4 + (lrow >> 1)) & kSwMask)) << 4);
         const unsigned grp_lds = uniform(my_lds + i * T * kTileBytes);
         static_for<T>([&](auto t) {
             dma16_at<true, t() * kTileRowBytes, t() * kTileBytes>(wbase, off0, grp_lds);
