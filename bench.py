@@ -201,7 +201,10 @@ def bench_gemm(torch, lib, steps: int, warmup: int):
     return ev_ms, wall_ms, kernel, kern_ms, median_ms
 
 
-def bench_decode(torch, lib, steps: int, warmup: int, shapes=None):
+def bench_decode(torch, lib, steps: int, warmup: int, shapes=None, activations: str = "normal", runs: int = 3):
+    """Per-launch time of back-to-back launches over rotating weights.  `activations`: "normal"
+    (clamp(round(N(0, 2))), the decode configuration) or "uniform"; `runs`: how many runs of
+    (warm-up, 300 timed launches), the median one being the figure."""
     import ctypes
 
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
@@ -210,19 +213,20 @@ def bench_decode(torch, lib, steps: int, warmup: int, shapes=None):
     for (m, n, k) in (shapes or DECODE_SHAPES):
         wbytes = n * k // 2
         nsets = max(4 if wbytes < (256 << 20) else 2, (768 << 20) // wbytes + 1)   # rotate through > 768 MiB of weights
-        x = packed_normal(torch, m, k, 31)   # activations: clamp(round(normal(0, 2))), weights uniform
+        # activations: clamp(round(normal(0, 2))) unless asked otherwise; weights uniform
+        x = packed_normal(torch, m, k, 31) if activations == "normal" else packed_random(torch, m, k, 31)
         sets = [(x, packed_random(torch, n, k, 40 + i), torch.empty((m, n), dtype=torch.int32, device="cuda"))
                 for i in range(nsets)]
         args = [(a.data_ptr(), b.data_ptr(), c.data_ptr(), m, n, k, stream) for (a, b, c) in sets]
 
-        # three runs of (warm-up, 300 timed launches); the median run is the figure, all three are listed
-        runs = sorted(time_launches(torch, (gemm, "int4linear_gemm_s4s4s32"), args, max(steps, 300), max(warmup, 20))[0]
-                      for _ in range(3))
-        ev_ms = runs[1]
+        # runs of (warm-up, 300 timed launches); the median run is the figure, all are listed
+        times = sorted(time_launches(torch, (gemm, "int4linear_gemm_s4s4s32"), args, max(steps, 300), max(warmup, 20))[0]
+                       for _ in range(runs))
+        ev_ms = times[len(times) // 2]
         algo_bytes = m * k // 2 + n * k // 2 + 4 * m * n
         gbs = algo_bytes / (ev_ms * 1e-3) / 1e9
         out.append({"shape": [m, n, k], "kernel": lib.kernel_for_shape(m, n, k), "us_per_launch": ev_ms * 1e3,
-                    "us_per_launch_runs": [round(r * 1e3, 3) for r in runs],
+                    "us_per_launch_runs": [round(r * 1e3, 3) for r in times],
                     "bytes": algo_bytes, "GB/s": gbs, "frac_of_hbm_peak": gbs / HBM_PEAK_GBS})
         del sets
         torch.cuda.empty_cache()
@@ -337,18 +341,39 @@ def cpu_baseline(budget_s: float = 15.0):
             "single_thread_sample": f"{rows1} rows, {dt1:.1f} s, oracle_linear_ref"}
 
 
+TRAFFIC_PROFILE = ROOT / "profiles" / "fp6_gemm_8192_and_decode_hbm_traffic.md"
+KERNEL_SOURCE = {"fp6": ROOT / "int4linear_amd" / "csrc" / "kernels_fp6.hip"}
+
+
+def source_digest(path: Path) -> str:
+    import hashlib
+
+    return hashlib.sha256(path.read_bytes()).hexdigest()
+
+
 def measured_traffic(kernel: str):
-    """HBM bytes per launch of the GEMM kernel as recorded from rocprofv3 counter runs
-    (FETCH_SIZE and WRITE_SIZE, each scaled by a plain copy of known size), or None."""
-    f = ROOT / "profiles" / "fp6_gemm_8192_and_decode_hbm_traffic.md"
-    if f.exists():
-        for line in f.read_text().splitlines():
-            if line.startswith(f"bytes_per_launch {kernel}_gemm_8192:"):
-                try:
-                    return int(line.split(":")[1])
-                except ValueError:
-                    return None
-    return None
+    """(HBM bytes per launch of the GEMM kernel, where the figure comes from).  The figure was
+    recorded from rocprofv3 counter runs (FETCH_SIZE and WRITE_SIZE, each scaled by a plain
+    copy of known size) together with a digest of the kernel's source file; it is reported only
+    while that file is still the one that was measured, otherwise None."""
+    if not TRAFFIC_PROFILE.exists() or kernel not in KERNEL_SOURCE:
+        return None, "no counter run on record for this kernel"
+    value = digest = None
+    for line in TRAFFIC_PROFILE.read_text().splitlines():
+        if line.startswith(f"bytes_per_launch {kernel}_gemm_8192:"):
+            try:
+                value = int(line.split(":")[1])
+            except ValueError:
+                value = None
+        if line.startswith(f"source_sha256 {KERNEL_SOURCE[kernel].name}:"):
+            digest = line.split(":")[1].strip()
+    where = f"rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs recorded in profiles/{TRAFFIC_PROFILE.name}"
+    if value is None:
+        return None, "no figure in " + where
+    if digest != source_digest(KERNEL_SOURCE[kernel]):
+        return None, (f"{KERNEL_SOURCE[kernel].name} has changed since the {where}: "
+                      "the recorded figure is withheld until the counters are read again")
+    return value, "static: " + where + " for this very source file, not measured by this run"
 
 
 def main() -> int:
@@ -398,6 +423,7 @@ def main() -> int:
     kernel_name = {"fp6": "fp6_gemm_kernel (v_mfma_f32_32x32x64_f8f6f4, E2M3 operands)",
                    "mfma": "mfma_gemm_kernel (v_mfma_i32_32x32x32_i8)"}.get(kernel, kernel)
 
+    traffic, traffic_source = measured_traffic(kernel)
     result = {
         "metric": "INT4 GEMM TOPS at M=N=K=8192 (% int8 MFMA peak); GB/s at M=16 decode",
         "value": tops_wall,
@@ -424,9 +450,8 @@ def main() -> int:
         "pct_of_int8_mfma_peak": 100.0 * tops_wall / INT8_MFMA_PEAK_TOPS,
         "roofline": {"bound": "mfma", "achieved": tops_kernel, "peak": peak,
                      "unit": "TFLOP/s", "frac": tops_kernel / peak,
-                     "traffic": measured_traffic(kernel),
-                     "traffic_source": "static: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs recorded in "
-                                       "profiles/fp6_gemm_8192_and_decode_hbm_traffic.md, not measured by this run",
+                     "traffic": traffic,
+                     "traffic_source": traffic_source,
                      "kernel": kernel_name,
                      "note": "2*M*N*K multiply-adds per launch / mean duration of the GEMM kernel itself: a HIP "
                              "event pair around each of its launches on caller-owned converted operands, in the "
@@ -443,6 +468,11 @@ def main() -> int:
         result["decode_note"] = ("mean time per launch of 300 back-to-back launches over rotating weights (> 768 MiB), median of three such runs; "
                                  "bare_stream_*: a kernel that only streams the same bytes in the same pattern, "
                                  "launched the same way (tests/host/stream_ceiling.cpp)")
+        # The statistic of this benchmark's first version, kept so that figures stay comparable
+        # across versions of the kernels: uniform activations, one run, the mean over the two
+        # large M = 16 shapes.
+        first = bench_decode(torch, lib, args.steps, args.warmup, DECODE_SHAPES[1:], activations="uniform", runs=1)
+        result["decode_GB/s_M16_uniform_activations_two_large_shapes"] = sum(d["GB/s"] for d in first) / len(first)
         result["decode_other_M"] = bench_decode(torch, lib, args.steps, args.warmup, DECODE_OTHER_M)
         if not args.no_extra:
             result["decode_large_W"] = bench_decode(torch, lib, args.steps, args.warmup, DECODE_LARGE_W)

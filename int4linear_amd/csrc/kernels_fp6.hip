@@ -244,21 +244,23 @@ struct Fp6Config {
     static_assert(CHUNKS % NWAVES == 0 && CH % 2 == 0 && CH <= 63, "loads must split evenly");
 };
 
-// Parts of the kernel that a measurement build leaves out to see what they cost
-// (tests/host/fp6_ablation.cpp instantiates them; the library only ever launches kWhole).
-// The results of such a build are wrong by construction.
-enum : unsigned {
-    kWhole = 0,
-    kNoStores = 1,    // the tile is not stored
-    kNoLoads = 2,     // no global -> LDS loads after the prologue (the ring keeps its first stages)
-    kNoLdsReads = 4,  // no LDS reads after the prologue (the registers keep their first operands)
-    kSameTile = 8,    // every tile reads the operands of tile (0, 0)
-    kNoBarrier = 16,  // the waves do not meet between a stage's two units (they then race on the ring)
+// What the GEMM kernel is put together from.  The library builds WholeKernel and nothing else;
+// tests/host/fp6_ablation.cpp, which compiles this file again, passes variations of its own
+// (derived from this one, with single members changed) to time what each part costs.
+struct WholeKernel {
+    static constexpr bool kStores = true;    // a finished tile is stored
+    static constexpr bool kLoads = true;     // global -> LDS loads go on after the prologue
+    static constexpr bool kLdsReads = true;  // LDS -> register reads go on after the prologue
+    static constexpr bool kOwnTile = true;   // a tile reads its own operands (false: those of tile (0, 0), L2-resident)
+    static constexpr bool kStagger = true;   // workgroups of an XCD start in groups (see the kernel)
+    static constexpr bool kFences = true;    // every MFMA and its share of the housekeeping are fenced off from the scheduler
+    // Called by lane 0 of wave 0 when the workgroup starts and after its last tile.
+    __device__ static void stamp(const Epilogue &, int /* workgroup */, int /* 0: start, 1: end */) {}
 };
 
 // HALF_OUT: the build for the two output kinds of 16-bit elements (its own build, so that the
 // one for 32-bit elements carries none of its code).
-template <class C, unsigned LEFT_OUT = kWhole, bool HALF_OUT = false>
+template <class C, bool HALF_OUT = false, class Parts = WholeKernel>
 __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
     const uint8_t *__restrict__ XW, const uint8_t *__restrict__ WW, int32_t *__restrict__ Y,
     int M, int N, int K, int tiles_m, int tiles_n, int ksplit, Epilogue ep)
@@ -302,7 +304,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
         const int item = bid + it * nblk;
         const int slice = item / tiles;
         tile_coords(item - slice * tiles, tiles, tiles_m, tiles_n, tm, tn);
-        if constexpr (LEFT_OUT & kSameTile)
+        if constexpr (!Parts::kOwnTile)
             tm = tn = 0;
         xptr = XW + ((size_t)tm * KT_all + (size_t)slice * KT) * kOperandStageBytes;
         wptr = WW + ((size_t)tn * KT_all + (size_t)slice * KT) * kOperandStageBytes;
@@ -392,9 +394,11 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
                 // down to its next use, past the housekeeping meant to run in its shadow;
                 // this empty statement "uses" the result here and keeps the MFMA in place.
                 pin(acc[i][j]);
-                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (Parts::kFences)
+                    __builtin_amdgcn_sched_barrier(0);
                 hook(std::integral_constant<int, SLOT>{});
-                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (Parts::kFences)
+                    __builtin_amdgcn_sched_barrier(0);
             }(), ...);
         }(std::make_integer_sequence<int, C::SLOTS>{});
     };
@@ -408,12 +412,12 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
     static_assert(kDmaFirstSlot + C::CH / 2 <= C::SLOTS, "not enough slots for the loads");
     auto spread = [&](auto slot_tag, unsigned read_ring, int read_kf, int read_p, auto half_pos, unsigned load_ring) {
         constexpr int slot = decltype(slot_tag)::value;
-        if constexpr (!(LEFT_OUT & kNoLdsReads)) {
+        if constexpr (Parts::kLdsReads) {
 #pragma unroll
             for (int r = slot * kReadsPerSlot; r < (slot + 1) * kReadsPerSlot && r < kReads; ++r)
                 read_op(read_ring, read_kf, read_p, r);
         }
-        if constexpr (!(LEFT_OUT & kNoLoads) && slot >= kDmaFirstSlot && slot < kDmaFirstSlot + C::CH / 2) {
+        if constexpr (Parts::kLoads && slot >= kDmaFirstSlot && slot < kDmaFirstSlot + C::CH / 2) {
             ld_chunk(std::integral_constant<int, decltype(half_pos)::value * (C::CH / 2) + slot - kDmaFirstSlot>{}, load_ring);
         }
     };
@@ -425,7 +429,9 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
     // far apart for the rest of the launch, which costs the spread once at the end and
     // saves most of the wait at every tile end before.  (The wait sits behind the first loads,
     // which travel meanwhile.)
-    if (total_tiles >= kStaggerMinRounds * nblk) {
+    if (threadIdx.x == 0)
+        Parts::stamp(ep, bid, 0);
+    if (Parts::kStagger && total_tiles >= kStaggerMinRounds * nblk) {
         const int grp = (bid >> 3) & (kStaggerGroups - 1);
         const unsigned long long until = wall_clock64() + (unsigned long long)(grp * kStaggerTicks);
         while (wall_clock64() < until)
@@ -440,7 +446,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
 #pragma unroll
     for (int r = 0; r < kReads; ++r)
         read_op(0u, 0, 0, r);
-    if constexpr (LEFT_OUT & kNoLdsReads) {
+    if constexpr (!Parts::kLdsReads) {
 #pragma unroll
         for (int r = 0; r < kReads; ++r)
             read_op(0u, 1, 1, r);
@@ -493,8 +499,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
                          : "scc", "memory");
             stores_behind = 0;
             __builtin_amdgcn_s_waitcnt(I4L_WAIT_LGKM0);
-            if constexpr (!(LEFT_OUT & kNoBarrier))
-                __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
         }
 
@@ -534,7 +539,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
                 const int ncol = ln + i * kFragRows;
                 col_off[i] = ncol < cols_left ? (unsigned)ncol * 4u : 0x40000000u;
             }
-            if constexpr (LEFT_OUT & kNoStores) {
+            if constexpr (!Parts::kStores) {
                 pin(acc[0][0]);
             } else if (ep_plain) {
 #pragma unroll
@@ -627,6 +632,8 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void fp6_gemm_kernel(
         if (iteration(std::integral_constant<int, 2>{}))
             break;
     }
+    if (threadIdx.x == 0)
+        Parts::stamp(ep, bid, 1);
 }
 
 // Eight wavefronts of 64 (m) x 128 (n), two per SIMD, one workgroup per CU.  (With four
@@ -681,7 +688,7 @@ hipError_t fp6_init(const DeviceInfo &dev)
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
     if (e != hipSuccess)
         return e;
-    return hipFuncSetAttribute((const void *)fp6_gemm_kernel<Fp6Cfg, kWhole, true>,
+    return hipFuncSetAttribute((const void *)fp6_gemm_kernel<Fp6Cfg, true>,
                                hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
 }
 
@@ -738,7 +745,7 @@ hipError_t launch_gemm_items(const void *a_conv, const void *b_conv, void *c, in
     if (ep.out >= kOutF16) {
         if (ksplit != 1)
             return hipErrorInvalidValue;
-        fp6_gemm_kernel<C, kWhole, true><<<(unsigned)grid, C::THREADS, kLdsBytes, stream>>>(
+        fp6_gemm_kernel<C, true><<<(unsigned)grid, C::THREADS, kLdsBytes, stream>>>(
             (const uint8_t *)a_conv, (const uint8_t *)b_conv, (int32_t *)c, m, n, padded_k(k), tiles_m, tiles_n, ksplit, ep);
     } else {
         fp6_gemm_kernel<C><<<(unsigned)grid, C::THREADS, kLdsBytes, stream>>>(

@@ -72,6 +72,7 @@ __device__ __forceinline__ int opaque(int v)
 
 // Marks a value as used (and possibly changed) at this point of the program.
 __device__ __forceinline__ void keep(v4i &v) { asm volatile("" : "+v"(v)); }
+__device__ __forceinline__ void keep(const v16i &v) { asm volatile("" ::"v"(v)); }
 
 constexpr int kStoreAux = 2;  // nt: C is written once and not read back by this kernel
 
@@ -132,7 +133,18 @@ __device__ __forceinline__ void tile_coords(int v, int total, int tiles_m, int t
     tn = in_group / gsz;
 }
 
-template <class C>
+// What mfma_gemm_kernel is put together from.  The library builds WholeInt8Kernel and nothing
+// else; tests/host/int8_ablation.cpp, which compiles this file again, passes variations of
+// its own (derived from this one, with single members changed) to time what each part costs.
+struct WholeInt8Kernel {
+    static constexpr bool kStores = true;    // a finished tile is stored
+    static constexpr bool kLoads = true;     // global -> LDS loads go on after the prologue
+    static constexpr bool kLdsReads = true;  // LDS -> register reads go on after the prologue
+    static constexpr bool kWiden = true;     // nibbles are widened to bytes between the MFMAs (false: the first operands stay)
+    static constexpr bool kStagger = true;   // workgroups of an XCD start in groups
+};
+
+template <class C, class Parts = WholeInt8Kernel>
 __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
     const uint8_t *__restrict__ X, const uint8_t *__restrict__ W, int32_t *__restrict__ Y,
     int M, int N, int K, int tiles_m, int tiles_n, int ksplit, Epilogue ep)
@@ -162,7 +174,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
     // mod 8) start in eight groups 0.8 us apart instead (measured: 4096 x 8192 x 1024 runs
     // 20 % faster, 8192^3 2 %; with the 128 x 128 tiles the spread costs more than it saves).
     if constexpr (C::BM == 256 && C::BN == 256) {
-        if (total_tiles >= 2 * nblk) {
+        if (Parts::kStagger && total_tiles >= 2 * nblk) {
             const int grp = (bid >> 3) & 7;
             const unsigned long long until = wall_clock64() + (unsigned long long)(grp * 80);  // 10-ns ticks
             while (wall_clock64() < until)
@@ -335,7 +347,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
                     acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(xhi[j % 2], whi[h][i], acc[i][j], 0, 0, 0);
                 constexpr int op0 = slot * n_ops / kSlots, op1 = (slot + 1) * n_ops / kSlots;
 #pragma unroll
-                for (int op = op0; op < op1; ++op) {
+                for (int op = op0; op < (Parts::kWiden ? op1 : op0); ++op) {
                     if (op < 12) {
                         widen_op(op, next_x, xlo[(j + 1) % 2], xhi[(j + 1) % 2]);
                     } else {
@@ -414,12 +426,12 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
         constexpr int pos = decltype(j_tag)::value * kSlots + decltype(slot_tag)::value;
 #pragma unroll
         for (int part = 0; part < kReadParts; ++part)
-            if (pos == part * kPositions / kReadParts + 1)
+            if (Parts::kLdsReads && pos == part * kPositions / kReadParts + 1)
                 read_part(read_ring, read_h, part, pk_w[read_h], pk_x[read_h]);
         constexpr int off = kDmaStride / 2;
         if constexpr (pos >= off && (pos - off) % kDmaStride == 0) {
             constexpr int idx = (pos - off) / kDmaStride;  // 0 .. CH-1
-            if (do_load && wave_par == idx % 2)
+            if (Parts::kLoads && do_load && wave_par == idx % 2)
                 ld_chunk(half_pos * (C::CH / 2) + idx / 2);
         }
     };
@@ -509,7 +521,13 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
                 const int ncol = ln + i * kFrag;
                 col_off[i] = ncol < cols_left ? (unsigned)ncol * 4u : 0x40000000u;
             }
-            if (ep_plain) {
+            if constexpr (!Parts::kStores) {
+#pragma unroll
+                for (int i = 0; i < C::FN; ++i)
+#pragma unroll
+                    for (int j = 0; j < C::FM; ++j)
+                        keep(acc[i][j]);  // (every accumulator counts as used: no MFMA may be dropped)
+            } else if (ep_plain) {
 #pragma unroll
                 for (int j = 0; j < C::FM; ++j) {
 #pragma unroll

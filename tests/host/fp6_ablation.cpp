@@ -1,15 +1,17 @@
 // Where the time of the FP6 GEMM kernel goes: the library's own kernel source compiled here
-// with parts of it left out (its LEFT_OUT template argument), every build timed on the same
-// converted operands.  What remains without stores, without global -> LDS loads and without
-// LDS reads is the MFMA loop with its barrier; each part's cost is the difference.  The
-// builds with parts left out compute nothing useful and their output is never looked at.
+// with variations of its WholeKernel description that leave single parts out, every build timed
+// on the same converted operands.  What remains without stores, without global -> LDS loads and
+// without LDS reads is the MFMA loop with its barrier; each part's cost is the difference.  The
+// builds with parts left out compute nothing useful and their output is never looked at.  One
+// more build keeps everything and records when every workgroup starts and ends, which gives the
+// spread of the ends and what the staggered start costs.
 //
 //   fp6_ablation [MxNxK] [--iters I] [--warmup W]       (default 8192x8192x8192, 40, 20)
 //
 // prints one line per build:  [ABLATION] <build> <us per launch> us <TOPS> TOPS
-// Run it under  rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES GRBM_GUI_ACTIVE  for the clock and the
-// share of cycles the matrix pipes are busy (the kernels differ in their last template
-// argument).
+// and one [SPREAD] line.  Run it under  rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES GRBM_GUI_ACTIVE
+// for the clock and the share of cycles the matrix pipes are busy (the kernels differ in their
+// last template argument).
 #include "../../int4linear_amd/csrc/kernels_fp6.hip"
 
 #include <cstdio>
@@ -41,17 +43,34 @@ __global__ void fill_kernel(uint32_t *p, size_t n, uint32_t seed)
     }
 }
 
-struct Build {
-    const char *name;
-    unsigned left_out;
+using int4linear::WholeKernel;
+struct SameTile : WholeKernel { static constexpr bool kOwnTile = false; };
+struct NoStores : WholeKernel { static constexpr bool kStores = false; };
+struct NoLdsReads : WholeKernel { static constexpr bool kLdsReads = false; };
+struct NoLoads : WholeKernel { static constexpr bool kLoads = false; };
+struct NoLoadsNoReads : NoLoads { static constexpr bool kLdsReads = false; };
+struct MfmaLoop : NoLoadsNoReads { static constexpr bool kStores = false; };            // MFMAs, barrier, loop
+struct MfmaLoopNoStagger : MfmaLoop { static constexpr bool kStagger = false; };
+struct MfmaLoopNoFences : MfmaLoop { static constexpr bool kFences = false; };
+struct MfmaLoopBare : MfmaLoop { static constexpr bool kStagger = false, kFences = false; };
+struct NoStagger : WholeKernel { static constexpr bool kStagger = false; };
+struct NoFences : WholeKernel { static constexpr bool kFences = false; };
+// The whole kernel with time stamps: the epilogue's bias pointer (unused: the launch passes an
+// epilogue that the kernel takes for "plain" only because `out` is 0 and the scales are null)
+// cannot carry them, so they go to a global the harness reads back.
+__device__ unsigned long long g_stamps[2][1024];
+struct Stamped : WholeKernel {
+    __device__ static void stamp(const int4linear::Epilogue &, int workgroup, int which) { g_stamps[which][workgroup & 1023] = wall_clock64(); }
 };
+struct StampedNoStagger : Stamped { static constexpr bool kStagger = false; };
+struct StampedMfmaLoop : StampedNoStagger { static constexpr bool kLoads = false, kLdsReads = false, kStores = false; };
 
-template <unsigned LEFT_OUT>
+template <class Parts>
 double time_build(const uint8_t *xw, const uint8_t *ww, int32_t *y, int m, int n, int k, int cus, int iters, int warmup)
 {
     using namespace int4linear;
     using C = Fp6Cfg;
-    auto kern = fp6_gemm_kernel<C, LEFT_OUT>;
+    auto kern = fp6_gemm_kernel<C, false, Parts>;
     CHECK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes));
     const int tiles_m = (m + kTileRows - 1) / kTileRows, tiles_n = (n + kTileRows - 1) / kTileRows;
     long grid = (long)cus * C::OCC;
@@ -74,6 +93,37 @@ double time_build(const uint8_t *xw, const uint8_t *ww, int32_t *y, int m, int n
     CHECK(hipEventDestroy(e0));
     CHECK(hipEventDestroy(e1));
     return (double)ms * 1e3 / iters;
+}
+
+// Start and end of every workgroup of the last launch, from the constant 100 MHz clock.
+void report_spread(const char *name, int workgroups)
+{
+    static unsigned long long h[2][1024];
+    CHECK(hipMemcpyFromSymbol(h, HIP_SYMBOL(g_stamps), sizeof h));
+    if (workgroups > 1024)
+        workgroups = 1024;
+    unsigned long long s0 = ~0ull, s1 = 0, e0 = ~0ull, e1 = 0;
+    for (int i = 0; i < workgroups; ++i) {
+        s0 = h[0][i] < s0 ? h[0][i] : s0;
+        s1 = h[0][i] > s1 ? h[0][i] : s1;
+        e0 = h[1][i] < e0 ? h[1][i] : e0;
+        e1 = h[1][i] > e1 ? h[1][i] : e1;
+    }
+    // workgroup ids go round the eight XCDs: the ends per XCD show whether the spread is between XCDs or inside them
+    for (int x = 0; x < 8 && x < workgroups; ++x) {
+        unsigned long long lo = ~0ull, hi = 0, sum = 0;
+        int cnt = 0;
+        for (int i = x; i < workgroups; i += 8, ++cnt) {
+            lo = h[1][i] < lo ? h[1][i] : lo;
+            hi = h[1][i] > hi ? h[1][i] : hi;
+            sum += h[1][i] - s0;
+        }
+        std::printf("[SPREAD-XCD] %-18s xcd %d: ends %7.2f .. %7.2f us after the first start (mean %7.2f)\n", name, x, (double)(lo - s0) / 100.0,
+                    (double)(hi - s0) / 100.0, (double)sum / cnt / 100.0);
+    }
+    std::printf("[SPREAD] %-22s first start to last start %6.2f us, first end to last end %6.2f us, first start to last end %7.2f us\n", name,
+                (double)(s1 - s0) / 100.0, (double)(e1 - e0) / 100.0, (double)(e1 - s0) / 100.0);
+    std::fflush(stdout);
 }
 
 }  // namespace
@@ -125,18 +175,26 @@ int main(int argc, char **argv)
         std::fflush(stdout);
     };
     // a load on the device before the first timed build, so that all of them meet the same clocks
-    time_build<kWhole>(xw, ww, y, m, n, k, cus, iters, warmup);
-    report("whole kernel", time_build<kWhole>(xw, ww, y, m, n, k, cus, iters, warmup));
-    report("every tile reads tile (0, 0)", time_build<kSameTile>(xw, ww, y, m, n, k, cus, iters, warmup));
-    report("no stores", time_build<kNoStores>(xw, ww, y, m, n, k, cus, iters, warmup));
-    report("no LDS reads", time_build<kNoLdsReads>(xw, ww, y, m, n, k, cus, iters, warmup));
-    report("no global -> LDS loads", time_build<kNoLoads>(xw, ww, y, m, n, k, cus, iters, warmup));
-    report("no loads, no LDS reads", time_build<kNoLoads | kNoLdsReads>(xw, ww, y, m, n, k, cus, iters, warmup));
-    report("no loads, no LDS reads, no stores (MFMA loop)",
-           time_build<kNoLoads | kNoLdsReads | kNoStores>(xw, ww, y, m, n, k, cus, iters, warmup));
-    report("the same without the barrier",
-           time_build<kNoLoads | kNoLdsReads | kNoStores | kNoBarrier>(xw, ww, y, m, n, k, cus, iters, warmup));
-    report("whole kernel without the barrier (racing)", time_build<kNoBarrier>(xw, ww, y, m, n, k, cus, iters, warmup));
-    report("whole kernel again", time_build<kWhole>(xw, ww, y, m, n, k, cus, iters, warmup));
+    time_build<WholeKernel>(xw, ww, y, m, n, k, cus, iters, warmup);
+    report("whole kernel", time_build<WholeKernel>(xw, ww, y, m, n, k, cus, iters, warmup));
+    report("every tile reads tile (0, 0)", time_build<SameTile>(xw, ww, y, m, n, k, cus, iters, warmup));
+    report("no stores", time_build<NoStores>(xw, ww, y, m, n, k, cus, iters, warmup));
+    report("no LDS reads", time_build<NoLdsReads>(xw, ww, y, m, n, k, cus, iters, warmup));
+    report("no global -> LDS loads", time_build<NoLoads>(xw, ww, y, m, n, k, cus, iters, warmup));
+    report("no loads, no LDS reads", time_build<NoLoadsNoReads>(xw, ww, y, m, n, k, cus, iters, warmup));
+    report("no staggered start", time_build<NoStagger>(xw, ww, y, m, n, k, cus, iters, warmup));
+    report("no scheduling fences", time_build<NoFences>(xw, ww, y, m, n, k, cus, iters, warmup));
+    report("MFMA loop (no loads, LDS reads, stores)", time_build<MfmaLoop>(xw, ww, y, m, n, k, cus, iters, warmup));
+    report("MFMA loop, no staggered start", time_build<MfmaLoopNoStagger>(xw, ww, y, m, n, k, cus, iters, warmup));
+    report("MFMA loop, no scheduling fences", time_build<MfmaLoopNoFences>(xw, ww, y, m, n, k, cus, iters, warmup));
+    report("MFMA loop, neither", time_build<MfmaLoopBare>(xw, ww, y, m, n, k, cus, iters, warmup));
+    report("whole kernel again", time_build<WholeKernel>(xw, ww, y, m, n, k, cus, iters, warmup));
+    const int tiles = ((m + kTileRows - 1) / kTileRows) * ((n + kTileRows - 1) / kTileRows);
+    report("whole kernel with time stamps", time_build<Stamped>(xw, ww, y, m, n, k, cus, iters, warmup));
+    report_spread("staggered start", tiles < cus ? tiles : cus);
+    report("no staggered start, with time stamps", time_build<StampedNoStagger>(xw, ww, y, m, n, k, cus, iters, warmup));
+    report_spread("all at once", tiles < cus ? tiles : cus);
+    report("MFMA loop, no staggered start, with time stamps", time_build<StampedMfmaLoop>(xw, ww, y, m, n, k, cus, iters, warmup));
+    report_spread("MFMA loop", tiles < cus ? tiles : cus);
     return 0;
 }

@@ -124,5 +124,22 @@ def test_fp6_ablation_reports_every_build(gpu):
                        capture_output=True, text=True, timeout=120)
     assert r.returncode == 0, r.stdout + r.stderr
     rows = re.findall(r"\[ABLATION\] (.*?) +([\d.]+) us +([\d.]+) TOPS", r.stdout)
-    assert len(rows) == 10 and rows[0][0] == "whole kernel", r.stdout
+    assert len(rows) == 16 and rows[0][0] == "whole kernel", r.stdout
+    assert r.stdout.count("[SPREAD]") == 3, r.stdout
+    assert all(float(us) > 0 and float(tops) > 0 for _, us, tops in rows), r.stdout
+
+
+def test_int8_ablation_usage_error_without_a_device():
+    r = subprocess.run([str(_binary("int8_ablation")), "--bogus"], capture_output=True, text=True)
+    assert r.returncode == 2 and "usage" in r.stderr
+
+
+@pytest.mark.gpu
+def test_int8_ablation_reports_every_build(gpu):
+    """The int8 kernel with parts left out: every build runs and reports a time."""
+    r = subprocess.run([str(_binary("int8_ablation")), "2048x2048x4096", "--iters", "10", "--warmup", "5"],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout + r.stderr
+    rows = re.findall(r"\[ABLATION\] (.*?) +([\d.]+) us +([\d.]+) TOPS", r.stdout)
+    assert len(rows) == 11 and rows[0][0] == "whole kernel", r.stdout
     assert all(float(us) > 0 and float(tops) > 0 for _, us, tops in rows), r.stdout
