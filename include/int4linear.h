@@ -22,8 +22,8 @@
  * handler).  With the limit set to 0 no entry point allocates anything.  Besides that the
  * library's device image holds the fixed scratch array of int4linear_gemm_s4s4s32_static
  * (INT4LINEAR_STATIC_SCRATCH_BYTES, 128 MiB of device memory on every device a process
- * initialises the library on, whether or not that entry point is ever called) and 64 KiB
- * of counters.
+ * initialises the library on, whether or not that entry point is ever called) and 32 KiB
+ * of arrival counters.
  *
  * HIP graphs: the first call on a device sets the library up (device queries, kernel
  * attributes, the address of the scratch array), which must not happen inside a capture:
