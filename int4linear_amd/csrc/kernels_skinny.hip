@@ -1,8 +1,9 @@
 // Weight-streaming kernels for skinny M: the decode-shaped linear layer.  Three kernels:
-// skinny_kernel (up to 64 rows of X per launch, W's rows split over one workgroup per CU),
-// skinny_stream_kernel (very many rows of W: workgroups that stay on their
-// CU) and skinny_basic_kernel (K that is not a whole number
-// of 128-byte tiles).
+// skinny_kernel (up to 64 rows of X per launch, W's rows split over one workgroup per CU;
+// as skinny_ksplit_kernel the same code with K split over workgroups as well, for 33 to 64
+// rows of X against long K), skinny_stream_kernel (very many rows of W: workgroups that
+// stay on their CU) and skinny_basic_kernel (K that is not a whole number of 128-byte
+// tiles).
 //
 // The job is HBM-bound: every byte of W (N x K/2) is read exactly once and the arithmetic
 // (v_mfma_i32_16x16x64_i8 after the same 16x nibble widening as the big int8 kernel:
@@ -32,8 +33,9 @@
 // loads) and adds its share to the group's block of sums in LDS without waiting for
 // anything; the waves meet once, at the end, and store the blocks side by side.  Each wave
 // fetches its own slice of X once and reuses it for its R row groups, so larger R cuts the
-// (L2-resident, but hot-line) X traffic.  No global atomics, no workspace, and the result
-// does not depend on timing (integer additions commute).
+// (L2-resident, but hot-line) X traffic.  No workspace (the form split over K apart), no
+// atomic operations on data, and the result does not depend on timing (integer additions
+// commute).
 #include "kernels.h"
 
 #include <utility>
