@@ -718,6 +718,36 @@ def test_random_shapes_against_the_scalar_kernel(gpu, seed):
         assert torch.equal(got, ref), f"shape {(m, n, k)} kernel {lib.kernel_for_shape(m, n, k)}"
 
 
+def test_random_decode_split_shapes_against_the_scalar_kernel(gpu):
+    """Random shapes in and around the regime in which the weight-streaming kernel splits K across
+    workgroups (33 to 64 rows of X, long K, up to 64 rows of W per quarter of the CUs), every
+    shape twice in a row (the arrival counters must be back at zero), whole outputs compared on
+    the device with the scalar kernel."""
+    import torch
+
+    import int4linear_amd as lib
+
+    rng = np.random.default_rng(20261)
+    g = torch.Generator(device="cuda:0")
+    split = 0
+    for _ in range(24):
+        m = int(rng.integers(30, 65))
+        n = int(rng.integers(200, 4300))
+        k = int(rng.choice([14336, 15360, 16384, 20480, 28672, 12288, 14336 + 256]))
+        split += lib.workspace_bytes(m, n, k) > 0
+        g.manual_seed(m * 1000003 + n * 101 + k)
+        x = torch.randint(0, 256, (m * k // 2,), dtype=torch.uint8, device="cuda:0", generator=g)
+        w = torch.randint(0, 256, (n * k // 2,), dtype=torch.uint8, device="cuda:0", generator=g)
+        ref = torch.full((m, n), -1, dtype=torch.int32, device="cuda:0")
+        lib.gemm_s4s4s32(x, w, ref, m, n, k, kernel="simple")
+        for rep in range(2):
+            got = torch.full((m, n), 0x5A5A5A5A, dtype=torch.int32, device="cuda:0")
+            lib.gemm_s4s4s32(x, w, got, m, n, k)
+            torch.cuda.synchronize()
+            assert torch.equal(got, ref), f"shape {(m, n, k)} call {rep} workspace {lib.workspace_bytes(m, n, k)}"
+    assert split >= 8, split  # the draw must actually reach the split form
+
+
 # ---- configuration 5: adversarial ---------------------------------------------------------
 
 def test_cfg5_all_minus_eight_full_size(gpu):
