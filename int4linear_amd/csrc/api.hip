@@ -344,7 +344,7 @@ int gemm_impl(const void *a, const void *b, void *c, int m, int n, int k, int ke
         kernel = pick_kernel(m, n, k, pd->info, limit);
         // A stream under capture gets the kernels that need no workspace.  Whether it is one
         // is asked only when the chosen kernel would touch the internal workspace or its
-        // ordering between streams: decode calls with up to 16 rows, a few microseconds
+        // ordering between streams: decode calls with up to 32 rows, a few microseconds
         // long, never pay for the query.
         if (source == Workspace::Internal &&
             (kernel == INT4LINEAR_KERNEL_FP6 ||
