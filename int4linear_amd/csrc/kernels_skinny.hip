@@ -554,6 +554,9 @@ __device__ __forceinline__ void skinny_body(const uint8_t *X, const uint8_t *W, 
         // stores them, and puts the counter back to zero for the next launch.  Nobody waits
         // for anybody; integer sums do not depend on who arrives when.  All of a wave's
         // operations of a kind go out together: a trip to memory costs far more than they do.
+        // (Release and acquire fences at device scope in place of the wait would say the same
+        // in the language's terms, but on this device they write back and invalidate the whole
+        // L2 of the XCD: measured 28 instead of 13 us for 64 x 4096 x 14336.)
         typedef unsigned long long u64;
         u64 *const slabs = (u64 *)partial + (size_t)row_block * kslices * kBlocks * 128 + lane;
         u64 *const mine_at = slabs + (size_t)kslice * kBlocks * 128;
