@@ -142,6 +142,8 @@ struct WholeInt8Kernel {
     static constexpr bool kLdsReads = true;  // LDS -> register reads go on after the prologue
     static constexpr bool kWiden = true;     // nibbles are widened to bytes between the MFMAs (false: the first operands stay)
     static constexpr bool kStagger = true;   // workgroups of an XCD start in groups
+    // Called by lane 0 of wave 0 when the workgroup starts and after its last tile.
+    __device__ static void stamp(int /* workgroup */, int /* 0: start, 1: end */) {}
 };
 
 template <class C, class Parts = WholeInt8Kernel>
@@ -168,6 +170,8 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
         return;
     const int my_tiles = (total_tiles - bid + nblk - 1) / nblk;
     const int total_stages = my_tiles * KT;
+    if (threadIdx.x == 0)
+        Parts::stamp(bid, 0);
     // Workgroups that start together reach every tile end together, and the stores of all
     // tiles then queue for the same path to memory while no CU computes.  With 256 x 256
     // tiles and two or more of them per workgroup, the workgroups of an XCD (ids congruent
@@ -610,6 +614,8 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void mfma_gemm_kernel(
     // The refills issued past the last stage must have landed before the workgroup's LDS
     // is handed to another one.
     __builtin_amdgcn_s_waitcnt(I4L_VMCNT(0));
+    if (threadIdx.x == 0)
+        Parts::stamp(bid, 1);
 }
 
 // ---- the form for grids of a few tiles per CU -----------------------------------------

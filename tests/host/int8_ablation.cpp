@@ -6,6 +6,7 @@
 //   int8_ablation [MxNxK] [--iters I] [--warmup W]       (default 8192x8192x8192, 30, 15)
 //
 // prints one line per build:  [ABLATION] <build> <us per launch> us <TOPS> TOPS
+// and, for two builds with time stamps, when the workgroups of every XCD end ([SPREAD-XCD]).
 // Run it under  rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES GRBM_GUI_ACTIVE  for the clock and the
 // share of cycles the matrix pipes are busy (the kernels differ in their last template
 // argument).
@@ -49,6 +50,12 @@ struct NoLoadsNoReads : NoLoads { static constexpr bool kLdsReads = false; };
 struct WidenAndMfma : NoLoadsNoReads { static constexpr bool kStores = false; };   // widening, MFMAs, barrier, loop
 struct MfmaLoop : WidenAndMfma { static constexpr bool kWiden = false; };           // MFMAs, barrier, loop
 struct MfmaLoopNoStagger : MfmaLoop { static constexpr bool kStagger = false; };
+// Builds that record when every workgroup starts and ends (the constant 100 MHz clock).
+__device__ unsigned long long g_stamps[2][1024];
+struct Stamped : WholeInt8Kernel {
+    __device__ static void stamp(int workgroup, int which) { g_stamps[which][workgroup & 1023] = wall_clock64(); }
+};
+struct StampedMfmaLoop : Stamped { static constexpr bool kLoads = false, kLdsReads = false, kStores = false, kWiden = false, kStagger = false; };
 
 template <class Parts>
 double time_build(const uint8_t *a, const uint8_t *b, int32_t *y, int m, int n, int k, int cus, int iters, int warmup)
@@ -78,6 +85,33 @@ double time_build(const uint8_t *a, const uint8_t *b, int32_t *y, int m, int n, 
     CHECK(hipEventDestroy(e0));
     CHECK(hipEventDestroy(e1));
     return (double)ms * 1e3 / iters;
+}
+
+// Start and end of every workgroup of the last launch, per XCD (workgroup ids go round the eight XCDs).
+void report_spread(const char *name, int workgroups)
+{
+    static unsigned long long h[2][1024];
+    CHECK(hipMemcpyFromSymbol(h, HIP_SYMBOL(g_stamps), sizeof h));
+    if (workgroups > 1024)
+        workgroups = 1024;
+    unsigned long long s0 = ~0ull, e0 = ~0ull, e1 = 0;
+    for (int i = 0; i < workgroups; ++i) {
+        s0 = h[0][i] < s0 ? h[0][i] : s0;
+        e0 = h[1][i] < e0 ? h[1][i] : e0;
+        e1 = h[1][i] > e1 ? h[1][i] : e1;
+    }
+    for (int x = 0; x < 8 && x < workgroups; ++x) {
+        unsigned long long lo = ~0ull, hi = 0;
+        for (int i = x; i < workgroups; i += 8) {
+            lo = h[1][i] < lo ? h[1][i] : lo;
+            hi = h[1][i] > hi ? h[1][i] : hi;
+        }
+        std::printf("[SPREAD-XCD] %-18s xcd %d: ends %7.2f .. %7.2f us after the first start\n", name, x, (double)(lo - s0) / 100.0,
+                    (double)(hi - s0) / 100.0);
+    }
+    std::printf("[SPREAD] %-22s first end to last end %6.2f us, first start to last end %7.2f us\n", name, (double)(e1 - e0) / 100.0,
+                (double)(e1 - s0) / 100.0);
+    std::fflush(stdout);
 }
 
 }  // namespace
@@ -137,5 +171,10 @@ int main(int argc, char **argv)
     report("MFMA loop (nothing else)", time_build<MfmaLoop>(a, b, y, m, n, k, cus, iters, warmup));
     report("MFMA loop, no staggered start", time_build<MfmaLoopNoStagger>(a, b, y, m, n, k, cus, iters, warmup));
     report("whole kernel again", time_build<WholeInt8Kernel>(a, b, y, m, n, k, cus, iters, warmup));
+    const int tiles = ((m + CfgLarge::BM - 1) / CfgLarge::BM) * ((n + CfgLarge::BN - 1) / CfgLarge::BN);
+    report("whole kernel with time stamps", time_build<Stamped>(a, b, y, m, n, k, cus, iters, warmup));
+    report_spread("whole kernel", tiles < cus ? tiles : cus);
+    report("MFMA loop, no staggered start, with time stamps", time_build<StampedMfmaLoop>(a, b, y, m, n, k, cus, iters, warmup));
+    report_spread("MFMA loop", tiles < cus ? tiles : cus);
     return 0;
 }

@@ -141,5 +141,6 @@ def test_int8_ablation_reports_every_build(gpu):
                        capture_output=True, text=True, timeout=120)
     assert r.returncode == 0, r.stdout + r.stderr
     rows = re.findall(r"\[ABLATION\] (.*?) +([\d.]+) us +([\d.]+) TOPS", r.stdout)
-    assert len(rows) == 11 and rows[0][0] == "whole kernel", r.stdout
+    assert len(rows) == 13 and rows[0][0] == "whole kernel", r.stdout
     assert all(float(us) > 0 and float(tops) > 0 for _, us, tops in rows), r.stdout
+    assert r.stdout.count("[SPREAD]") == 2, r.stdout
