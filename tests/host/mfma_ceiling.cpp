@@ -1,7 +1,8 @@
 // What the matrix pipes sustain with nothing else going on: loops of nothing but MFMAs on
 // operands held in registers, for the two instructions the library's large-shape kernels issue
 // (v_mfma_i32_32x32x32_i8 and v_mfma_f32_32x32x64_f8f6f4 with FP6 E2M3 operands), on operand
-// data of several kinds.  The rate depends on the data: at the device's power limit the clock
+// data of several kinds, among them every exact encoding of signed 4-bit values that the FP6 / BF6
+// formats offer (the one the FP6 kernel uses, n/8 in E2M3, draws the least power of them).  The rate depends on the data: at the device's power limit the clock
 // drops as more operand bits toggle, so "peak" is reached on zeros only.  Each line gives the
 // throughput, the shader clock observed while the loop ran (cycle counter against the constant
 // 100 MHz counter) and the share of the launch's cycles the matrix pipes were busy (32 cycles
@@ -9,7 +10,7 @@
 // against; the reference has no counterpart (its README quotes no peak, README.md:57-62).
 //
 //   mfma_ceiling [--iters N]
-//   prints lines:  [MFMA] <int8|fp6> <data> <TOPS> TOPS <GHz> GHz <busy %>
+//   prints lines:  [MFMA] <int8|fp6|bf6> <data> <TOPS> TOPS <GHz> GHz <busy %>
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -39,7 +40,23 @@ __device__ unsigned mix(unsigned x)
     return x;
 }
 
-enum Data { kZeros = 0, kRandom = 1, kNibbleTimes16 = 2, kSignExtendedS4 = 3, kS4Codes = 4 };
+enum Data {
+    kZeros = 0, kRandom = 1, kNibbleTimes16 = 2, kSignExtendedS4 = 3,
+    // Exact codes of uniform s4 values n: E2M3 n/8 (the FP6 kernel's), n/4, n/2; E3M2 n and n/16.
+    kS4Codes = 4, kS4CodesQuarter = 5, kS4CodesHalf = 6, kBf6CodesOne = 7, kBf6CodesSixteenth = 8
+};
+
+// The magnitude bits (exponent and mantissa) of |n| = mg in the given exact encoding.
+__device__ unsigned s4_magnitude_code(int data, unsigned mg)
+{
+    if (data == kS4Codes) return mg;                                  // E2M3, n/8: subnormals up to 7/8, then 1.0
+    if (data == kS4CodesQuarter) return mg << 1;                       // E2M3, n/4
+    if (data == kS4CodesHalf) return mg <= 4 ? mg << 2 : 2 * mg + 8;   // E2M3, n/2
+    if (mg == 0) return 0;
+    const int lg = 31 - __builtin_clz(mg);                             // mg = 2^lg * 1.ff
+    const int ex = lg + 3 + (data == kBf6CodesOne ? 0 : -4);           // E3M2, bias 3
+    return ex >= 1 ? ((unsigned)ex << 2) | (((mg << 2) >> lg) & 3u) : mg;   // below 4/16: subnormal mg/16
+}
 
 // One dword of int8 operand data of the given kind.
 __device__ unsigned int8_word(int data, unsigned r)
@@ -53,17 +70,17 @@ __device__ unsigned int8_word(int data, unsigned r)
     return r;
 }
 
-// 32 FP6 values (192 bits) for one lane: random bits, or E2M3 codes of uniform s4 values
-// (sign << 5 | magnitude: what the FP6 kernel's converter writes).
+// 32 six-bit values (192 bits) for one lane: random bits, or codes of uniform s4 values
+// (sign << 5 | magnitude; kS4Codes is what the FP6 kernel's converter writes).
 __device__ v8i fp6_operand(int data, unsigned seed)
 {
     unsigned w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     if (data == kRandom)
         for (int i = 0; i < 6; ++i) w[i] = mix(seed + i);
-    if (data == kS4Codes)
+    if (data >= kS4Codes)
         for (int e = 0; e < 32; ++e) {
             const int n = (int)(mix(seed + 100 + e) & 15u) - 8;
-            const unsigned code = (n < 0 ? 32u : 0u) | (unsigned)(n < 0 ? -n : n);
+            const unsigned code = (n < 0 ? 32u : 0u) | s4_magnitude_code(data, (unsigned)(n < 0 ? -n : n));
             const int bit = 6 * e;
             w[bit >> 5] |= code << (bit & 31);
             if ((bit & 31) > 26) w[(bit >> 5) + 1] |= code >> (32 - (bit & 31));
@@ -72,7 +89,8 @@ __device__ v8i fp6_operand(int data, unsigned seed)
 }
 
 // cycles[0] = shader cycles, cycles[1] = 100 MHz ticks of the loop, as seen by wave 0 of block 0
-template <bool FP6>
+// FMT: the instruction's operand format field (2 = E2M3, 3 = E3M2)
+template <bool FP6, int FMT = 2>
 __global__ __launch_bounds__(512) void mfma_loop(int *out, long long *cycles, int iters, int data)
 {
     const unsigned seed = (threadIdx.x + blockIdx.x * 512u) * 2654435761u;
@@ -87,7 +105,7 @@ __global__ __launch_bounds__(512) void mfma_loop(int *out, long long *cycles, in
         for (int it = 0; it < iters; ++it) {
 #pragma unroll
             for (int i = 0; i < 8; ++i)
-                acc[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[i & 3], b[(i + (i >> 2)) & 3], acc[i], 2, 2, 0, 0, 0, 0);
+                acc[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[i & 3], b[(i + (i >> 2)) & 3], acc[i], FMT, FMT, 0, 0, 0, 0);
         }
         c1 = __builtin_readcyclecounter(); r1 = __builtin_amdgcn_s_memrealtime();
         for (int i = 0; i < 8; ++i) for (int j = 0; j < 16; ++j) sum += (int)acc[i][j];
@@ -112,7 +130,7 @@ __global__ __launch_bounds__(512) void mfma_loop(int *out, long long *cycles, in
     if (blockIdx.x == 0 && threadIdx.x == 0) { cycles[0] = c1 - c0; cycles[1] = r1 - r0; }
 }
 
-template <bool FP6>
+template <bool FP6, int FMT = 2>
 void run(const char *kind, const char *name, int data, int iters, int cus, int *out, long long *cycles_d)
 {
     hipEvent_t e0, e1;
@@ -120,10 +138,10 @@ void run(const char *kind, const char *name, int data, int iters, int cus, int *
     HIP_OK(hipEventCreate(&e1));
     const int launches = 20;
     // untimed: lets the clock settle under this load
-    for (int l = 0; l < launches; ++l) mfma_loop<FP6><<<cus, 512>>>(out, cycles_d, iters, data);
+    for (int l = 0; l < launches; ++l) mfma_loop<FP6, FMT><<<cus, 512>>>(out, cycles_d, iters, data);
     HIP_OK(hipDeviceSynchronize());
     HIP_OK(hipEventRecord(e0));
-    for (int l = 0; l < launches; ++l) mfma_loop<FP6><<<cus, 512>>>(out, cycles_d, iters, data);
+    for (int l = 0; l < launches; ++l) mfma_loop<FP6, FMT><<<cus, 512>>>(out, cycles_d, iters, data);
     HIP_OK(hipEventRecord(e1));
     HIP_OK(hipEventSynchronize(e1));
     float ms = 0;
@@ -165,6 +183,11 @@ int main(int argc, char **argv)
     run<true>("fp6", "zeros", kZeros, iters, cus, out, cycles);
     run<true>("fp6", "random-bits", kRandom, iters, cus, out, cycles);
     run<true>("fp6", "s4-codes (kernel's form)", kS4Codes, iters, cus, out, cycles);
+    // the other exact encodings of s4 values the instruction offers
+    run<true>("fp6", "s4-codes n/4 (E2M3)", kS4CodesQuarter, iters, cus, out, cycles);
+    run<true>("fp6", "s4-codes n/2 (E2M3)", kS4CodesHalf, iters, cus, out, cycles);
+    run<true, 3>("bf6", "s4-codes n (E3M2)", kBf6CodesOne, iters, cus, out, cycles);
+    run<true, 3>("bf6", "s4-codes n/16 (E3M2)", kBf6CodesSixteenth, iters, cus, out, cycles);
     run<false>("int8", "zeros-again", kZeros, iters, cus, out, cycles);
     return 0;
 }

@@ -106,8 +106,8 @@ def test_mfma_ceiling_usage_error_without_a_device():
 def test_mfma_ceiling_reports_rates(gpu):
     r = subprocess.run([str(_binary("mfma_ceiling")), "--iters", "500"], capture_output=True, text=True, timeout=120)
     assert r.returncode == 0, r.stdout + r.stderr
-    rows = re.findall(r"\[MFMA\] (int8|fp6) .*? ([\d.]+) TOPS +([\d.]+) GHz", r.stdout)
-    assert len(rows) == 8 and all(float(t) > 500 and 0.5 < float(g) < 3.0 for _, t, g in rows), r.stdout
+    rows = re.findall(r"\[MFMA\] (int8|fp6|bf6) .*? ([\d.]+) TOPS +([\d.]+) GHz", r.stdout)
+    assert len(rows) == 12 and all(float(t) > 500 and 0.5 < float(g) < 3.0 for _, t, g in rows), r.stdout
 
 
 def test_fp6_ablation_usage_error_without_a_device():
