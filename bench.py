@@ -18,6 +18,8 @@ One JSON line is printed.  Besides the whole-run figure it carries
                 type it issues,
   decode        the skinny-M weight-streaming kernel at M = 16 against HBM bandwidth,
   cpu_baseline  the CPU oracle's loop nest timed on this host's cores on a row sample,
+  static_weights  the same problem with W converted once beforehand, as a linear layer with static
+                weights would run it (per step: convert X, then the GEMM on converted operands),
   int8_kernel   the same 8192^3 problem on the library's int8-MFMA kernel (the path that
                 needs no workspace), against the int8 MFMA dense peak,
   vendor        hipBLASLt's int8 GEMM on the widened operands, timed by the C++ harness
@@ -172,9 +174,10 @@ def bench_gemm(torch, lib, steps: int, warmup: int):
     # The dominant kernel's own duration inside the same sequence of kernels as the timed
     # region: each step converts both operands into caller-owned buffers (what the call above
     # does into the library's workspace) and then runs the FP6 GEMM between a pair of HIP
-    # events on the stream it is launched on.  (Timed in a loop of nothing but GEMMs the
-    # kernel runs 8-10 % slower: the device's power limit then holds the clock lower than
-    # in the real sequence, where the memory-bound converter sits between two GEMMs.)
+    # events on the stream it is launched on.  (Timed in a loop of nothing but GEMMs on
+    # operands converted beforehand the kernel runs 8-10 % slower: rotating operand sets then
+    # come from HBM instead of the memory-side cache the converter has just left them in, and
+    # without the memory-bound converter between two GEMMs the power limit holds the clock lower.)
     kernel = lib.kernel_for_shape(M, N, K)
     kern_ms = ev_ms
     if kernel == "fp6":
@@ -285,6 +288,45 @@ def bench_int8_kernel(torch, lib, steps: int, warmup: int):
     tops = 2.0 * M * N * K / (ev_ms * 1e-3) / 1e12
     return {"kernel": "mfma_gemm_kernel (v_mfma_i32_32x32x32_i8)", "kernel_ms": ev_ms, "TOPS": tops,
             "frac_of_int8_peak": tops / INT8_MFMA_PEAK_TOPS}
+
+
+def bench_static_weights(torch, lib, steps: int, warmup: int):
+    """The 8192^3 problem the way a linear layer with static weights would run it: W converted
+    once before the timed region (int4linear_fp6_convert), every step converts the activations
+    X and multiplies (int4linear_gemm_fp6_converted).  Reported beside `value`, never as it:
+    `value` converts both operands in every call, as the reference's entry point implies."""
+    import ctypes
+
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    convert = raw_entry("int4linear_fp6_convert")
+    gemm6 = raw_entry("int4linear_gemm_fp6_converted")
+    sets = []
+    for s in range(3):
+        a = packed_random(torch, M, K, 3000 + s)
+        b = packed_random(torch, N, K, 4000 + s)
+        ac = torch.empty(lib.fp6_operand_bytes(M, K), dtype=torch.uint8, device="cuda")
+        bc = torch.empty(lib.fp6_operand_bytes(N, K), dtype=torch.uint8, device="cuda")
+        c = torch.empty((M, N), dtype=torch.int32, device="cuda")
+        if convert(b.data_ptr(), bc.data_ptr(), N, K, stream) != 0:
+            raise RuntimeError("int4linear_fp6_convert failed")
+        sets.append((a, ac, bc, c))
+        del b
+    torch.cuda.synchronize()
+
+    def launch(t):
+        a, ac, bc, c = t
+        st = convert(a.data_ptr(), ac.data_ptr(), M, K, stream)
+        st |= gemm6(ac.data_ptr(), bc.data_ptr(), c.data_ptr(), M, N, K, stream)
+        if st != 0:
+            raise RuntimeError(f"the caller-owned FP6 entry points failed (status bits {st})")
+
+    ramp_clocks(torch, launch, sets)
+    ev_ms, _ = time_launches(torch, launch, sets, steps, warmup)
+    return {"what": "W converted once beforehand (int4linear_fp6_convert), per step: convert X, int4linear_gemm_fp6_converted",
+            "ms_per_step": ev_ms, "TOPS": 2.0 * M * N * K / (ev_ms * 1e-3) / 1e12,
+            "note": "three sets of operands rotate, so the converted W comes from HBM in every step; the per-call "
+                    "converter of the default path leaves it in the memory-side cache instead, which at this size is "
+                    "worth about what the conversion costs"}
 
 
 def vendor_line():
@@ -481,6 +523,8 @@ def main() -> int:
         if not args.no_ceiling:
             add_ceilings(all_dec, stream_ceilings([tuple(d["shape"]) for d in all_dec]))
     if not args.no_extra:
+        if kernel == "fp6":
+            result["static_weights"] = bench_static_weights(torch, lib, max(10, args.steps // 2), args.warmup)
         result["int8_kernel"] = bench_int8_kernel(torch, lib, max(10, args.steps // 2), args.warmup)
         if not args.no_vendor:
             result["vendor"] = vendor_line()
